@@ -1,0 +1,81 @@
+// Shared device/host helpers for the gfx950 kernels: bf16 bit handling, MFMA operand types,
+// error plumbing of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdexcept>
+#include <string>
+
+typedef uint16_t bf16_t; // raw bf16 bits in memory
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// native vectors for 16/8-byte memory accesses (HIP's uint4/uint2 structs copy through memcpy,
+// which keeps register arrays of them in scratch memory)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define TG_DEVICE __device__ __forceinline__
+
+TG_DEVICE float bf16_to_float(bf16_t b) {
+    return __uint_as_float(uint32_t(b) << 16);
+}
+// round to nearest even (v_cvt_pk_bf16_f32 on gfx950)
+TG_DEVICE bf16_t float_to_bf16(float f) {
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+TG_DEVICE uint32_t pack_bf16(float lo, float hi) {
+    return uint32_t(float_to_bf16(lo)) | (uint32_t(float_to_bf16(hi)) << 16);
+}
+TG_DEVICE float bf16_lo(uint32_t pair) {
+    return __uint_as_float(pair << 16);
+}
+TG_DEVICE float bf16_hi(uint32_t pair) {
+    return __uint_as_float(pair & 0xffff0000u);
+}
+TG_DEVICE float round_bf16(float f) {
+    return bf16_to_float(float_to_bf16(f));
+}
+// exact-erf GELU and its derivative
+TG_DEVICE float gelu_f(float x) {
+    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+}
+TG_DEVICE float gelu_grad_f(float x) {
+    return 0.5f * (1.0f + erff(x * 0.70710678118654752f)) +
+           x * 0.39894228040143268f * __expf(-0.5f * x * x);
+}
+TG_DEVICE float wave_sum(float x) {
+#pragma unroll
+    for (int k = 32; k; k >>= 1)
+        x += __shfl_xor(x, k, 64);
+    return x;
+}
+TG_DEVICE float wave_max(float x) {
+#pragma unroll
+    for (int k = 32; k; k >>= 1)
+        x = fmaxf(x, __shfl_xor(x, k, 64));
+    return x;
+}
+
+// ---- host side ---------------------------------------------------------------------------
+extern thread_local std::string tg_last_error;
+
+inline void check_hip(hipError_t error, const char *what = "") {
+    if (error != hipSuccess)
+        throw std::runtime_error(std::string(what) + hipGetErrorString(error));
+}
+inline void require(bool ok, const char *message) {
+    if (!ok)
+        throw std::invalid_argument(message);
+}
+// Every C entry point is `return guarded([&]{ ... });` : 0 on success, -1 with the message
+// kept for tg_error()/tgk_error(); no exception crosses the ABI.
+template <class F> inline int guarded(F &&body) {
+    try {
+        body();
+        return 0;
+    } catch (const std::exception &error) {
+        tg_last_error = error.what();
+        return -1;
+    }
+}
