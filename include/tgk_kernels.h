@@ -57,6 +57,24 @@ TGK_API int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uint16
                    size_t workspace_bytes);
 TGK_API size_t tgk_gemm_wgrad_workspace(int M, int N, int K);
 
+/* ---- Causal softmax attention, head_dim 64.  Takes the slot of attention_forward /
+ * attention_backward (cuda/attention.cuh:48-106); the reference's arg-max attention is replaced
+ * by softmax(Q K^T * scale + causal mask) V as the target specifies.  Layout is the reference's
+ * (cuda/attention.cuh:38-39,68): Q, K, V are [B*T][ld] views with head h at columns h*64..h*64+63
+ * (normally three column slices of the packed qkv buffer, ld = 3*d), O is [B*T][ldo].
+ * lse is [B][H][T] fp32 = natural log of the row sums of exp(scaled scores).
+ * T multiple of 128; pointers 16-byte aligned; leading dimensions multiples of 8. ---- */
+TGK_API int tgk_attn_fwd(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
+                         const uint16_t *K, const uint16_t *V, int ld, uint16_t *O, int ldo, float *lse,
+                         float scale);
+/* Recompute backward from Q, K, V, O, lse: dQ, dK, dV ([B*T][lddq] views, same head layout).
+ * Deterministic (no atomics).  workspace: tgk_attn_bwd_workspace(B,H,T) bytes. */
+TGK_API int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
+                         const uint16_t *K, const uint16_t *V, int ld, const uint16_t *O, int ldo,
+                         const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ, uint16_t *dK,
+                         uint16_t *dV, int lddq, float scale, void *workspace, size_t workspace_bytes);
+TGK_API size_t tgk_attn_bwd_workspace(int B, int H, int T);
+
 #ifdef __cplusplus
 }
 #endif

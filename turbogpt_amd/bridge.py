@@ -20,6 +20,10 @@ KERNEL_ABI = {
     "tgk_gemm_dgrad": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
     "tgk_gemm_wgrad": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, i32, vp, sz]),
     "tgk_gemm_wgrad_workspace": (sz, [i32, i32, i32]),
+    "tgk_attn_fwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, f32]),
+    "tgk_attn_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32,
+                           f32, vp, sz]),
+    "tgk_attn_bwd_workspace": (sz, [i32, i32, i32]),
 }
 ENGINE_ABI = {
     "tg_error": (C.c_char_p, []),

@@ -1,0 +1,478 @@
+// Causal softmax attention for gfx950, head_dim 64: flash-style forward (online softmax, fp32
+// log-sum-exp saved) and recompute backward.  Takes the slot of attention_forward /
+// attention_backward in the reference's layer (cuda/attention.cuh:48-106; called from
+// cuda/model.cuh:20 and :86-88); the packed [token][q|k|v] buffer and the [token][head*64+d]
+// output keep the reference's layout (cuda/attention.cuh:38-39,68), so no permutes are needed.
+//
+// All three kernels work on 32x32 MFMA tiles (v_mfma_f32_32x32x16_bf16) and are written in the
+// "transposed" form: the score tile is produced as S^T[key][query] so that one lane owns one
+// query row - row maxima / sums / rescales are per-lane scalars - and the fp32 accumulator
+// registers of S^T can be fed back, converted to bf16, as the B operand of the next product with
+// no cross-lane movement.  The operand that must then be read "k-strided" (V for P.V, K for dS.K,
+// Q and dO for the dK/dV products) is fetched with the transposing LDS read ds_read_b64_tr_b16.
+//
+// backward = three launches: delta = rowsum(dO o O); dK/dV (one block per 128 keys, loops over
+// query tiles); dQ (one block per 128 queries, loops over key tiles).  No atomics: every output
+// element has one owner and a fixed summation order, so results are bit-reproducible.
+#include "common.h"
+#include "../../include/tgk_kernels.h"
+
+namespace {
+
+constexpr int HD = 64;      // head dimension
+constexpr int LS = HD + 8;  // LDS row stride in elements
+constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+TG_DEVICE f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        z[r] = 0.f;
+    return z;
+}
+TG_DEVICE f32x16 mfma(bf16x8 rows_to_regs, bf16x8 rows_to_lanes, f32x16 acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_to_regs, rows_to_lanes, acc, 0, 0, 0);
+}
+// row index owned by accumulator register r of a 32x32 tile (lane half g = lane/32)
+TG_DEVICE int acc_row(int r, int g) {
+    return 8 * (r >> 2) + 4 * g + (r & 3);
+}
+// 16-byte fragment of a [row][k] LDS tile: row = row0 + lane%32, k = k0 + 8*(lane/32) .. +7
+TG_DEVICE bf16x8 frag_rows(const bf16_t *tile, int row0, int k0, int lane) {
+    return *reinterpret_cast<const bf16x8 *>(tile + (row0 + (lane & 31)) * LS + k0 + (lane >> 5) * 8);
+}
+// Fragment of the same tile read along its rows: the lane gets column col0 + lane%32 and the 8
+// rows  krow0 + 4g + {0..3}  and  krow0 + 8 + 4g + {0..3}  - exactly the rows that accumulator
+// registers 8*kk2 .. 8*kk2+7 of a 32x32 tile hold (acc_row), so a converted accumulator and this
+// fragment agree on the order of the reduced index.
+TG_DEVICE bf16x8 frag_cols(const bf16_t *tile, int krow0, int col0, int lane) {
+    const int g = lane >> 5, blk = (lane >> 4) & 1, i = lane & 15;
+    const bf16_t *p = tile + (krow0 + 4 * g + (i >> 2)) * LS + col0 + 16 * blk + 4 * (i & 3);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 8 * LS));
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, both);
+}
+// registers 8*kk2 .. 8*kk2+7 of an fp32 accumulator as a bf16 operand fragment
+TG_DEVICE bf16x8 acc_to_frag(const f32x16 &acc, int kk2) {
+    bf16x8 f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        f[j] = (__bf16)acc[8 * kk2 + j];
+    return f;
+}
+TG_DEVICE float exp2_fast(float x) {
+    return __builtin_amdgcn_exp2f(x);
+}
+
+// 64 rows x 64 columns of a [token][ld] bf16 matrix -> registers -> LDS tile, 256 threads
+TG_DEVICE void tile_load(u32x4 (&regs)[2], const bf16_t *base, int ld, int tid) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int c = tid + i * 256, row = c >> 3, kc = c & 7;
+        regs[i] = *reinterpret_cast<const u32x4 *>(base + size_t(row) * ld + kc * 8);
+    }
+}
+TG_DEVICE void tile_store(const u32x4 (&regs)[2], bf16_t *tile, int tid) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int c = tid + i * 256, row = c >> 3, kc = c & 7;
+        *reinterpret_cast<u32x4 *>(tile + row * LS + kc * 8) = regs[i];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward: block = 128 queries (4 waves x 32), key/value tiles of 64, heavy (late) tiles first
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const bf16_t *__restrict__ Q,
+                                                          const bf16_t *__restrict__ K,
+                                                          const bf16_t *__restrict__ V, int ld,
+                                                          bf16_t *__restrict__ O, int ldo,
+                                                          float *__restrict__ LSE, int T, int H,
+                                                          float c) {
+    __shared__ __align__(16) bf16_t sK[2][64 * LS], sV[2][64 * LS];
+    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5;
+    const int wave_q0 = q0 + wave * 32, qrow = wave_q0 + (lane & 31);
+    const size_t token0 = size_t(b) * T;
+
+    bf16x8 qf[4];
+    {
+        const bf16_t *qp = Q + (token0 + qrow) * ld + h * HD + g * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+            qf[ks] = *reinterpret_cast<const bf16x8 *>(qp + ks * 16);
+    }
+    f32x16 o[2] = {zero16(), zero16()};
+    float m = -INFINITY, l = 0.f;
+
+    const int tiles = (q0 + 128) / 64;
+    const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
+    u32x4 kr[2], vr[2];
+    tile_load(kr, kbase, ld, tid);
+    tile_load(vr, vbase, ld, tid);
+    tile_store(kr, sK[0], tid);
+    tile_store(vr, sV[0], tid);
+    __syncthreads();
+    for (int j = 0; j < tiles; ++j) {
+        const int cur = j & 1, kv0 = j * 64;
+        const bool more = j + 1 < tiles;
+        if (more) {
+            tile_load(kr, kbase + size_t(kv0 + 64) * ld, ld, tid);
+            tile_load(vr, vbase + size_t(kv0 + 64) * ld, ld, tid);
+        }
+        if (kv0 <= wave_q0 + 31) { // some key of this tile is visible to this wave (wave uniform)
+            f32x16 s[2] = {zero16(), zero16()};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+                    s[mt] = mfma(frag_rows(sK[cur], mt * 32, ks * 16, lane), qf[ks], s[mt]);
+            if (kv0 + 63 > wave_q0) { // diagonal tile: hide keys after the query
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (kv0 + mt * 32 + acc_row(r, g) > qrow)
+                            s[mt][r] = -INFINITY;
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    mx = fmaxf(mx, s[mt][r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx * c);
+            const float alpha = exp2_fast(m - m_new);
+            float sum = 0.f;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float p = exp2_fast(fmaf(s[mt][r], c, -m_new));
+                    s[mt][r] = p;
+                    sum += p;
+                }
+            sum += __shfl_xor(sum, 32, 64);
+            l = l * alpha + sum;
+            m = m_new;
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    o[dt][r] *= alpha;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const bf16x8 pf = acc_to_frag(s[kk >> 1], kk & 1);
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+                    o[dt] = mfma(frag_cols(sV[cur], kk * 16, dt * 32, lane), pf, o[dt]);
+            }
+        }
+        if (more) {
+            tile_store(kr, sK[cur ^ 1], tid);
+            tile_store(vr, sV[cur ^ 1], tid);
+        }
+        __syncthreads();
+    }
+    const float inv = 1.0f / l;
+    bf16_t *op = O + (token0 + qrow) * ldo + h * HD + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            u32x2 packed;
+            packed.x = pack_bf16(o[dt][q4 * 4 + 0] * inv, o[dt][q4 * 4 + 1] * inv);
+            packed.y = pack_bf16(o[dt][q4 * 4 + 2] * inv, o[dt][q4 * 4 + 3] * inv);
+            *reinterpret_cast<u32x2 *>(op + dt * 32 + q4 * 8) = packed;
+        }
+    if (g == 0)
+        LSE[(size_t(b) * H + h) * T + qrow] = (m + __log2f(l)) * LN2;
+}
+
+// delta[b][h][t] = sum_d dO[t][h*64+d] * O[t][h*64+d]; one 8-lane group per (token, head)
+__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *__restrict__ dO, int lddo,
+                                                         const bf16_t *__restrict__ O, int ldo,
+                                                         float *__restrict__ delta, int T, int H,
+                                                         int rows) {
+    const int idx = blockIdx.x * 32 + (threadIdx.x >> 3), part = threadIdx.x & 7;
+    if (idx >= rows * H)
+        return;
+    const int token = idx / H, h = idx - token * H;
+    const u32x4 a = *reinterpret_cast<const u32x4 *>(dO + size_t(token) * lddo + h * HD + part * 8);
+    const u32x4 o = *reinterpret_cast<const u32x4 *>(O + size_t(token) * ldo + h * HD + part * 8);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        sum += bf16_lo(a[i]) * bf16_lo(o[i]) + bf16_hi(a[i]) * bf16_hi(o[i]);
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    sum += __shfl_xor(sum, 4, 64);
+    if (part == 0) {
+        const int b = token / T, t = token - b * T;
+        delta[(size_t(b) * H + h) * T + t] = sum;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dK, dV: block = 128 keys (4 waves x 32), loops over 64-query tiles from the diagonal on.
+// Scores are produced as S[query][key] here: one lane owns one KEY, which is the row index of
+// both outputs.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
+    const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
+    const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ LSE,
+    const float *__restrict__ delta, bf16_t *__restrict__ dK, bf16_t *__restrict__ dV, int lddq, int T,
+    int H, float scale) {
+    __shared__ __align__(16) bf16_t sQ[2][64 * LS], sdO[2][64 * LS];
+    const int k0 = blockIdx.x * 128, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5;
+    const int wave_k0 = k0 + wave * 32, krow = wave_k0 + (lane & 31);
+    const size_t token0 = size_t(b) * T;
+    const float c = scale * LOG2E;
+
+    bf16x8 kf[4], vf[4];
+    {
+        const bf16_t *kp = K + (token0 + krow) * ld + h * HD + g * 8;
+        const bf16_t *vp = V + (token0 + krow) * ld + h * HD + g * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            kf[ks] = *reinterpret_cast<const bf16x8 *>(kp + ks * 16);
+            vf[ks] = *reinterpret_cast<const bf16x8 *>(vp + ks * 16);
+        }
+    }
+    f32x16 dk[2] = {zero16(), zero16()}, dv[2] = {zero16(), zero16()};
+    const float *lse_row = LSE + (size_t(b) * H + h) * T, *delta_row = delta + (size_t(b) * H + h) * T;
+
+    const int first = k0 / 64, tiles = T / 64;
+    const bf16_t *qbase = Q + token0 * ld + h * HD, *gbase = dO + token0 * lddo + h * HD;
+    u32x4 qr[2], gr[2];
+    tile_load(qr, qbase + size_t(first) * 64 * ld, ld, tid);
+    tile_load(gr, gbase + size_t(first) * 64 * lddo, lddo, tid);
+    tile_store(qr, sQ[0], tid);
+    tile_store(gr, sdO[0], tid);
+    __syncthreads();
+    for (int j = first; j < tiles; ++j) {
+        const int cur = (j - first) & 1, q0 = j * 64;
+        const bool more = j + 1 < tiles;
+        if (more) {
+            tile_load(qr, qbase + size_t(q0 + 64) * ld, ld, tid);
+            tile_load(gr, gbase + size_t(q0 + 64) * lddo, lddo, tid);
+        }
+        if (q0 + 63 >= wave_k0) { // some query of this tile sees this wave's keys (wave uniform)
+            f32x16 s[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt) {
+                    s[qt] = mfma(frag_rows(sQ[cur], qt * 32, ks * 16, lane), kf[ks], s[qt]);
+                    dp[qt] = mfma(frag_rows(sdO[cur], qt * 32, ks * 16, lane), vf[ks], dp[qt]);
+                }
+            const bool diagonal = q0 < wave_k0 + 31;
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const int q = q0 + qt * 32 + 8 * q4 + 4 * g;
+                    const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_row + q);
+                    const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_row + q);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = q4 * 4 + e;
+                        float p = exp2_fast(fmaf(s[qt][r], c, -lse4[e] * LOG2E));
+                        if (diagonal && krow > q + e)
+                            p = 0.f;
+                        s[qt][r] = p;
+                        dp[qt][r] = p * (dp[qt][r] - del4[e]);
+                    }
+                }
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const bf16x8 pf = acc_to_frag(s[kk >> 1], kk & 1);
+                const bf16x8 dsf = acc_to_frag(dp[kk >> 1], kk & 1);
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt) {
+                    dv[dt] = mfma(frag_cols(sdO[cur], kk * 16, dt * 32, lane), pf, dv[dt]);
+                    dk[dt] = mfma(frag_cols(sQ[cur], kk * 16, dt * 32, lane), dsf, dk[dt]);
+                }
+            }
+        }
+        if (more) {
+            tile_store(qr, sQ[cur ^ 1], tid);
+            tile_store(gr, sdO[cur ^ 1], tid);
+        }
+        __syncthreads();
+    }
+    bf16_t *kp = dK + (token0 + krow) * lddq + h * HD + 4 * g;
+    bf16_t *vp = dV + (token0 + krow) * lddq + h * HD + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            u32x2 pk, pv;
+            pk.x = pack_bf16(dk[dt][q4 * 4 + 0] * scale, dk[dt][q4 * 4 + 1] * scale);
+            pk.y = pack_bf16(dk[dt][q4 * 4 + 2] * scale, dk[dt][q4 * 4 + 3] * scale);
+            pv.x = pack_bf16(dv[dt][q4 * 4 + 0], dv[dt][q4 * 4 + 1]);
+            pv.y = pack_bf16(dv[dt][q4 * 4 + 2], dv[dt][q4 * 4 + 3]);
+            *reinterpret_cast<u32x2 *>(kp + dt * 32 + q4 * 8) = pk;
+            *reinterpret_cast<u32x2 *>(vp + dt * 32 + q4 * 8) = pv;
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dQ: block = 128 queries (4 waves x 32), loops over 64-key tiles up to the diagonal.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
+    const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
+    const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ LSE,
+    const float *__restrict__ delta, bf16_t *__restrict__ dQ, int lddq, int T, int H, float scale) {
+    __shared__ __align__(16) bf16_t sK[2][64 * LS], sV[2][64 * LS];
+    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128, h = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5;
+    const int wave_q0 = q0 + wave * 32, qrow = wave_q0 + (lane & 31);
+    const size_t token0 = size_t(b) * T;
+    const float c = scale * LOG2E;
+
+    bf16x8 qf[4], gf[4];
+    {
+        const bf16_t *qp = Q + (token0 + qrow) * ld + h * HD + g * 8;
+        const bf16_t *gp = dO + (token0 + qrow) * lddo + h * HD + g * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            qf[ks] = *reinterpret_cast<const bf16x8 *>(qp + ks * 16);
+            gf[ks] = *reinterpret_cast<const bf16x8 *>(gp + ks * 16);
+        }
+    }
+    const float lse2 = LSE[(size_t(b) * H + h) * T + qrow] * LOG2E;
+    const float del = delta[(size_t(b) * H + h) * T + qrow];
+    f32x16 dq[2] = {zero16(), zero16()};
+
+    const int tiles = (q0 + 128) / 64;
+    const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
+    u32x4 kr[2], vr[2];
+    tile_load(kr, kbase, ld, tid);
+    tile_load(vr, vbase, ld, tid);
+    tile_store(kr, sK[0], tid);
+    tile_store(vr, sV[0], tid);
+    __syncthreads();
+    for (int j = 0; j < tiles; ++j) {
+        const int cur = j & 1, kv0 = j * 64;
+        const bool more = j + 1 < tiles;
+        if (more) {
+            tile_load(kr, kbase + size_t(kv0 + 64) * ld, ld, tid);
+            tile_load(vr, vbase + size_t(kv0 + 64) * ld, ld, tid);
+        }
+        if (kv0 <= wave_q0 + 31) {
+            f32x16 s[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt) {
+                    s[mt] = mfma(frag_rows(sK[cur], mt * 32, ks * 16, lane), qf[ks], s[mt]);
+                    dp[mt] = mfma(frag_rows(sV[cur], mt * 32, ks * 16, lane), gf[ks], dp[mt]);
+                }
+            const bool diagonal = kv0 + 63 > wave_q0;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float p = exp2_fast(fmaf(s[mt][r], c, -lse2));
+                    if (diagonal && kv0 + mt * 32 + acc_row(r, g) > qrow)
+                        p = 0.f;
+                    dp[mt][r] = p * (dp[mt][r] - del);
+                }
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const bf16x8 dsf = acc_to_frag(dp[kk >> 1], kk & 1);
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+                    dq[dt] = mfma(frag_cols(sK[cur], kk * 16, dt * 32, lane), dsf, dq[dt]);
+            }
+        }
+        if (more) {
+            tile_store(kr, sK[cur ^ 1], tid);
+            tile_store(vr, sV[cur ^ 1], tid);
+        }
+        __syncthreads();
+    }
+    bf16_t *qp = dQ + (token0 + qrow) * lddq + h * HD + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            u32x2 packed;
+            packed.x = pack_bf16(dq[dt][q4 * 4 + 0] * scale, dq[dt][q4 * 4 + 1] * scale);
+            packed.y = pack_bf16(dq[dt][q4 * 4 + 2] * scale, dq[dt][q4 * 4 + 3] * scale);
+            *reinterpret_cast<u32x2 *>(qp + dt * 32 + q4 * 8) = packed;
+        }
+}
+
+void check_attention_shape(int B, int H, int T, int hd) {
+    require(B > 0 && H > 0 && T > 0, "attention: empty shape");
+    require(hd == HD, "attention: head_dim must be 64");
+    require(T % 128 == 0, "attention: context must be a multiple of 128");
+    require(size_t(B) * T < (size_t(1) << 31), "attention: too many tokens");
+}
+void check_matrix(const void *p, int ld, const char *name) {
+    if (!p || (reinterpret_cast<uintptr_t>(p) & 15) || ld % 8)
+        throw std::invalid_argument(std::string("attention operand ") + name +
+                                    " must be non-null, 16-byte aligned, leading dimension % 8 == 0");
+}
+
+} // namespace
+
+extern "C" int tgk_attn_fwd(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
+                            const uint16_t *K, const uint16_t *V, int ld, uint16_t *O, int ldo,
+                            float *lse, float scale) {
+    return guarded([&] {
+        check_attention_shape(B, H, T, hd);
+        check_matrix(Q, ld, "Q");
+        check_matrix(K, ld, "K");
+        check_matrix(V, ld, "V");
+        check_matrix(O, ldo, "O");
+        require(lse && !(reinterpret_cast<uintptr_t>(lse) & 15), "attention: lse must be 16-byte aligned");
+        hipLaunchKernelGGL(attn_fwd_kernel, dim3(T / 128, H, B), dim3(256), 0, stream, Q, K, V, ld, O, ldo,
+                           lse, T, H, scale * LOG2E);
+        check_hip(hipGetLastError(), "attention forward launch: ");
+    });
+}
+
+extern "C" size_t tgk_attn_bwd_workspace(int B, int H, int T) {
+    return size_t(B) * H * T * sizeof(float);
+}
+
+extern "C" int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
+                            const uint16_t *K, const uint16_t *V, int ld, const uint16_t *O, int ldo,
+                            const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ, uint16_t *dK,
+                            uint16_t *dV, int lddq, float scale, void *workspace,
+                            size_t workspace_bytes) {
+    return guarded([&] {
+        check_attention_shape(B, H, T, hd);
+        check_matrix(Q, ld, "Q");
+        check_matrix(K, ld, "K");
+        check_matrix(V, ld, "V");
+        check_matrix(O, ldo, "O");
+        check_matrix(dO, lddo, "dO");
+        check_matrix(dQ, lddq, "dQ");
+        check_matrix(dK, lddq, "dK");
+        check_matrix(dV, lddq, "dV");
+        require(lse && !(reinterpret_cast<uintptr_t>(lse) & 15), "attention: lse must be 16-byte aligned");
+        require(workspace && workspace_bytes >= tgk_attn_bwd_workspace(B, H, T) &&
+                    !(reinterpret_cast<uintptr_t>(workspace) & 15),
+                "attention backward: workspace too small (see tgk_attn_bwd_workspace)");
+        float *delta = static_cast<float *>(workspace);
+        const int rows = B * T;
+        hipLaunchKernelGGL(attn_delta_kernel, dim3((rows * H + 31) / 32), dim3(256), 0, stream, dO, lddo, O,
+                           ldo, delta, T, H, rows);
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel, dim3(T / 128, H, B), dim3(256), 0, stream, Q, K, V, ld, dO,
+                           lddo, lse, delta, dK, dV, lddq, T, H, scale);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3(T / 128, H, B), dim3(256), 0, stream, Q, K, V, ld, dO,
+                           lddo, lse, delta, dQ, lddq, T, H, scale);
+        check_hip(hipGetLastError(), "attention backward launch: ");
+    });
+}
