@@ -75,6 +75,61 @@ TGK_API int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, const 
                          uint16_t *dV, int lddq, float scale, void *workspace, size_t workspace_bytes);
 TGK_API size_t tgk_attn_bwd_workspace(int B, int H, int T);
 
+/* ---- HBM-bound operators.  Parameters are held as two 16-bit halves of their fp32 master:
+ * `hi` (the bf16 compute weight, truncated) and `lo` (cuda/ops.cuh:6-14); operators that need
+ * full fp32 parameters (norm scales) take both halves, as precise_weight does. ---- */
+
+/* out[t] = RN_bf16(table[x[t]] + positions[t % T]); replaces the gather of load_tile
+ * (cuda/dataset.cuh:31-32) and adds the learned positions the target model uses. */
+TGK_API int tgk_embed_fwd(hipStream_t stream, int rows, int T, int D, const uint8_t *x,
+                          const uint16_t *table, const uint16_t *positions, uint16_t *out);
+/* dtable[v] (=|+=) sum_{t: x[t]=v} dh[t]; dpositions[p] (=|+=) sum_b dh[b*T+p]; fp32.  Replaces
+ * the atomicAdd scatter of cuda/model.cuh:96-97 with a fixed-order sum. D multiple of 64. */
+TGK_API int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab, const uint8_t *x,
+                          const uint16_t *dh, float *dtable, float *dpositions, int accumulate);
+
+/* y = RN_bf16((x - mean) * rsqrt(var + eps) * gamma + beta) per row; takes the slot of normalize
+ * (cuda/ops.cuh:57-66; RMSNorm there, LayerNorm in the target model). D multiple of 8, <= 2048. */
+TGK_API int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint16_t *x,
+                              const uint16_t *gamma_hi, const uint16_t *gamma_lo,
+                              const uint16_t *beta_hi, const uint16_t *beta_lo, uint16_t *y, float eps);
+/* dx = RN_bf16(LN'(x) dy), or with residual != 0: dx = RN_bf16(dx + RN_bf16(LN'(x) dy)) (residual
+ * gradients stay in bf16, cuda/ops.cuh:74-76); dgamma/dbeta (=|+=) fixed-order column sums in
+ * fp32 (replaces the atomicAdd of cuda/ops.cuh:77).  Takes the slot of norm_backward
+ * (cuda/ops.cuh:67-80).  workspace: tgk_layernorm_bwd_workspace(rows, D) bytes. */
+TGK_API int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint16_t *x, const uint16_t *dy,
+                              const uint16_t *gamma_hi, const uint16_t *gamma_lo, uint16_t *dx,
+                              float *dgamma, float *dbeta, float eps, int residual, int accumulate,
+                              void *workspace, size_t workspace_bytes);
+TGK_API size_t tgk_layernorm_bwd_workspace(int rows, int D);
+
+/* Softmax cross-entropy over 256 byte classes on bf16 logits [rows][256] (cuda/model.cuh:33-58):
+ * loss[t] = logsumexp - logit[y[t]]; logits_f32 (optional) receives the logits as fp32;
+ * write_grad != 0 overwrites the logits with RN_bf16((softmax - onehot) * inv_count). */
+TGK_API int tgk_cross_entropy(hipStream_t stream, int rows, int vocab, uint16_t *logits, const uint8_t *y,
+                              float *loss, float *logits_f32, float inv_count, int write_grad);
+
+/* partials[i] = sum of squares of block i's share of g (cuda/trainer.cuh:35-46); count <= 4096. */
+TGK_API int tgk_sumsq_partials(hipStream_t stream, const float *g, size_t n, float *partials, int count);
+/* AdamW on the hi/lo weight halves (cuda/optim.cuh:67-106): clip scale min(1, clip/(||g||+1e-6))
+ * from the folded partials when clip > 0, m += (1-b1)(g-m), v = b2 v + (1-b2) g^2,
+ * w = w (1 - lr*wd) - (lr/bc1) m / (sqrt(v)/sqrt(bc2) + eps), bias corrections from `step`
+ * (0-based) with the current beta1.  segment_starts (device, sorted, first = 0) and
+ * segment_flags (device, bit 0 = apply weight decay) describe the decay groups
+ * (cuda/optim.cuh:5-15).  n and all segment starts multiples of 4. */
+TGK_API int tgk_adamw(hipStream_t stream, size_t n, uint16_t *weight_hi, uint16_t *weight_lo, float *m,
+                      float *v, const float *g, const float *norm_partials, int norm_count,
+                      const int64_t *segment_starts, const uint8_t *segment_flags, int segments, float lr,
+                      float beta1, float beta2, float eps, float weight_decay, float clip, uint64_t step);
+
+/* Hash-sampled batch (cuda/dataset.cuh:13-27): endpoint e = low + hash_u64(seed + step*batch + b)
+ * mod (size - low), low = max(8, context); x = data[e-context : e], y = data[e-context+1 : e+1]. */
+TGK_API int tgk_sample_batch(hipStream_t stream, const uint8_t *data, int64_t size, uint64_t seed,
+                             uint64_t step, int batch, int context, uint8_t *x, uint8_t *y);
+/* out[p] = mean over the batch of token_loss[b*context + p], in double (cuda/trainer.cuh:79-100). */
+TGK_API int tgk_position_means(hipStream_t stream, const float *token_loss, int batch, int context,
+                               float *out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,179 @@
+"""GPU parity of the HBM-bound operators (embedding, LayerNorm, cross-entropy, AdamW on hi/lo
+weights, sampling, loss means) against the CPU checker, through the C ABI.  bf16 outputs are held
+to relative L2 <= 1e-2 (and to agreement with the checker's bf16-rounding mode); fp32 outputs to
+1e-5; integer/byte results bit-exactly."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import check, host, library, rel, stream, sync, to_bf16_device
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a, dtype=None):
+    return torch.from_numpy(np.ascontiguousarray(a if dtype is None else a.astype(dtype))).cuda()
+
+
+def hilo(orc, w):
+    hi, lo = orc.split_hilo(w)
+    return dev(hi.view(np.int16)), dev(lo.view(np.int16))
+
+
+@pytest.mark.parametrize("B,T,D", [(2, 128, 256), (3, 64, 768)])
+def test_embedding_forward_and_backward(orc, B, T, D):
+    lib = library()
+    rng = np.random.default_rng(B + T + D)
+    table, th = to_bf16_device(rng.standard_normal((256, D)))
+    pos, ph = to_bf16_device(rng.standard_normal((T, D)))
+    x = orc.fill_zipf_bytes(B * T, 71)  # repeated symbols exercise the gather-sum
+    xd = dev(x)
+    out = torch.empty(B * T, D, dtype=torch.bfloat16, device="cuda")
+    check(lib.tgk_embed_fwd(stream(), B * T, T, D, xd.data_ptr(), table.data_ptr(), pos.data_ptr(), out.data_ptr()))
+    sync()
+    want = orc.bf16_round(th[x] + np.tile(ph, (B, 1)))
+    np.testing.assert_array_equal(host(out), want)
+    dh, dhh = to_bf16_device(rng.standard_normal((B * T, D)))
+    dt = torch.full((256, D), 1.0, dtype=torch.float32, device="cuda")
+    dp = torch.full((T, D), 1.0, dtype=torch.float32, device="cuda")
+    check(lib.tgk_embed_bwd(stream(), B, T, D, 256, xd.data_ptr(), dh.data_ptr(), dt.data_ptr(), dp.data_ptr(), 0))
+    sync()
+    want_t = np.zeros((256, D), np.float64)
+    np.add.at(want_t, x, dhh.astype(np.float64))
+    assert rel(host(dt), want_t) < 1e-6
+    assert rel(host(dp), dhh.reshape(B, T, D).astype(np.float64).sum(0)) < 1e-6
+    check(lib.tgk_embed_bwd(stream(), B, T, D, 256, xd.data_ptr(), dh.data_ptr(), dt.data_ptr(), dp.data_ptr(), 1))
+    sync()
+    assert rel(host(dt), 2 * want_t) < 1e-6
+
+
+@pytest.mark.parametrize("M,D", [(64, 256), (333, 768), (128, 1024), (16, 2048)])
+def test_layernorm_forward_backward(orc, M, D):
+    lib = library()
+    rng = np.random.default_rng(M + D)
+    x, xh = to_bf16_device(rng.standard_normal((M, D)) * 2 + 0.5)
+    dy, dyh = to_bf16_device(rng.standard_normal((M, D)))
+    gamma = (1 + 0.2 * rng.standard_normal(D)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(D)).astype(np.float32)
+    gh, gl = hilo(orc, gamma)
+    bh, bl = hilo(orc, beta)
+    y = torch.empty(M, D, dtype=torch.bfloat16, device="cuda")
+    check(lib.tgk_layernorm_fwd(stream(), M, D, x.data_ptr(), gh.data_ptr(), gl.data_ptr(), bh.data_ptr(),
+                                bl.data_ptr(), y.data_ptr(), 1e-5))
+    sync()
+    assert rel(host(y), orc.layernorm_fwd(xh, gamma, beta)) < 1e-2
+    assert np.mean(host(y) == orc.layernorm_fwd(xh, gamma, beta, emulate=True)) > 0.98
+    need = lib.tgk_layernorm_bwd_workspace(M, D)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    for residual in (0, 1):
+        prior, ph = to_bf16_device(rng.standard_normal((M, D)))
+        dx = prior.clone()
+        dg = torch.full((D,), 2.0, dtype=torch.float32, device="cuda")
+        db = torch.full((D,), 2.0, dtype=torch.float32, device="cuda")
+        check(lib.tgk_layernorm_bwd(stream(), M, D, x.data_ptr(), dy.data_ptr(), gh.data_ptr(), gl.data_ptr(),
+                                    dx.data_ptr(), dg.data_ptr(), db.data_ptr(), 1e-5, residual, residual,
+                                    ws.data_ptr(), need))
+        sync()
+        want_dx, want_dg, want_db = orc.layernorm_bwd(xh, dyh, gamma, dx_in=ph if residual else None)
+        assert rel(host(dx), want_dx) < 1e-2
+        base = 2.0 if residual else 0.0  # accumulate flag follows residual in this test
+        assert rel(host(dg) - base, want_dg) < 1e-4
+        assert rel(host(db) - base, want_db) < 1e-4
+
+
+def test_cross_entropy_loss_logits_and_gradient(orc):
+    lib = library()
+    rng = np.random.default_rng(17)
+    M = 1000
+    logits, lh = to_bf16_device(rng.standard_normal((M, 256)) * 3)
+    y = rng.integers(0, 256, M, dtype=np.uint8)
+    yd = dev(y)
+    loss = torch.empty(M, dtype=torch.float32, device="cuda")
+    f32 = torch.empty(M, 256, dtype=torch.float32, device="cuda")
+    work = logits.clone()
+    check(lib.tgk_cross_entropy(stream(), M, 256, work.data_ptr(), yd.data_ptr(), loss.data_ptr(), f32.data_ptr(),
+                                1.0 / M, 0))
+    sync()
+    want_loss, want_grad = orc.cross_entropy(lh, y)
+    np.testing.assert_allclose(host(loss), want_loss, rtol=1e-5, atol=1e-5)
+    np.testing.assert_array_equal(host(f32), lh)
+    assert torch.equal(work, logits)  # evaluation mode leaves the logits alone
+    check(lib.tgk_cross_entropy(stream(), M, 256, work.data_ptr(), yd.data_ptr(), loss.data_ptr(), None, 1.0 / M, 1))
+    sync()
+    assert rel(host(work), want_grad) < 1e-2
+    assert rel(host(work), orc.cross_entropy(lh, y, emulate=True)[1]) < 1e-3
+
+
+def run_adamw(orc, w, m, v, g, bounds, flags, steps, clip, lr=6e-4, wd=0.1):
+    lib = library()
+    n = w.size
+    hi, lo = hilo(orc, w)
+    md, vd = dev(m), dev(v)
+    bd, fd = dev(np.asarray(bounds, np.int64)), dev(np.asarray(flags, np.uint8))
+    parts = torch.empty(1024, dtype=torch.float32, device="cuda")
+    for step, grad in enumerate(g[:steps]):
+        gd = dev(grad)
+        check(lib.tgk_sumsq_partials(stream(), gd.data_ptr(), n, parts.data_ptr(), 1024))
+        check(lib.tgk_adamw(stream(), n, hi.data_ptr(), lo.data_ptr(), md.data_ptr(), vd.data_ptr(), gd.data_ptr(),
+                            parts.data_ptr(), 1024, bd.data_ptr(), fd.data_ptr(), len(bounds), lr, 0.9, 0.95, 1e-8,
+                            wd, clip, step))
+        sync()
+    out = orc.join_hilo(hi.cpu().numpy().view(np.uint16), lo.cpu().numpy().view(np.uint16))
+    return out, md.cpu().numpy(), vd.cpu().numpy()
+
+
+@pytest.mark.parametrize("clip", [0.0, 1.0])
+def test_adamw_matches_the_checker_over_20_steps(orc, clip):
+    # tests/verify.py:64-105 (AdamW part): N(0, 0.01) gradients from default_rng(192)
+    rng = np.random.default_rng(192)
+    n = 40960
+    bounds, flags = [0, 4096, 8192, 30000], [0, 1, 0, 1]
+    decay = np.zeros(n, np.uint8)
+    decay[4096:8192] = 1
+    decay[30000:] = 1
+    w0 = (rng.standard_normal(n) * 0.02).astype(np.float32)
+    grads = [(rng.standard_normal(n) * (0.01 if clip == 0 else 0.05)).astype(np.float32) for _ in range(20)]
+    got, gm, gv = run_adamw(orc, w0, np.zeros(n, np.float32), np.zeros(n, np.float32), grads, bounds, flags, 20, clip)
+    w, m, v = w0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for step, g in enumerate(grads):
+        w, m, v = orc.adamw(w, m, v, g, decay, 6e-4, 0.9, 0.95, 1e-8, 0.1, orc.clip_scale(g, clip), step)
+    assert rel(got - w0, w - w0) < 1e-4              # verify.py:101
+    np.testing.assert_allclose(got, w, atol=2e-6, rtol=2e-5)  # verify.py:103
+    np.testing.assert_allclose(gm, m, rtol=1e-4, atol=1e-9)
+    np.testing.assert_allclose(gv, v, rtol=1e-4, atol=1e-12)
+
+
+def test_adamw_keeps_updates_below_one_bf16_ulp(orc):
+    # tests/verify.py:108-127: w=.5, g=.01, lr=1e-5, 64 steps; plain bf16 would stall at .5
+    n = 4096
+    grads = [np.full(n, 0.01, np.float32)] * 64
+    got, _, _ = run_adamw(orc, np.full(n, 0.5, np.float32), np.zeros(n, np.float32), np.zeros(n, np.float32),
+                          grads, [0], [0], 64, 0.0, lr=1e-5, wd=0.0)
+    assert np.max(np.abs(got - 0.5)) > 5e-4
+    np.testing.assert_allclose(0.5 - got, 64e-5, rtol=0.02)
+    plain = torch.tensor(0.5, dtype=torch.bfloat16)
+    for _ in range(64):
+        plain -= 1e-5
+    assert plain.item() == 0.5
+
+
+def test_sampling_and_position_means_are_exact(orc):
+    lib = library()
+    data = orc.fill_zipf_bytes(100000, 71)
+    dd = dev(data)
+    for batch, context, step in [(16, 4, 0), (12, 8, 5), (16, 1024, 3)]:
+        x = torch.empty(batch, context, dtype=torch.uint8, device="cuda")
+        y = torch.empty_like(x)
+        check(lib.tgk_sample_batch(stream(), dd.data_ptr(), data.size, 3407, step, batch, context, x.data_ptr(),
+                                   y.data_ptr()))
+        sync()
+        wx, wy = orc.sample_batch(data, 3407, step, batch, context)
+        np.testing.assert_array_equal(x.cpu().numpy(), wx)
+        np.testing.assert_array_equal(y.cpu().numpy(), wy)
+    tl = np.random.default_rng(3).random((24, 256)).astype(np.float32)
+    out = torch.empty(256, dtype=torch.float32, device="cuda")
+    check(lib.tgk_position_means(stream(), dev(tl).data_ptr(), 24, 256, out.data_ptr()))
+    sync()
+    np.testing.assert_array_equal(host(out), (tl.astype(np.float64).sum(0) / 24).astype(np.float32))

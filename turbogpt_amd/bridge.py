@@ -24,6 +24,17 @@ KERNEL_ABI = {
     "tgk_attn_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32,
                            f32, vp, sz]),
     "tgk_attn_bwd_workspace": (sz, [i32, i32, i32]),
+    "tgk_embed_fwd": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
+    "tgk_embed_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32]),
+    "tgk_layernorm_fwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, f32]),
+    "tgk_layernorm_bwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, f32, i32, i32, vp, sz]),
+    "tgk_layernorm_bwd_workspace": (sz, [i32, i32]),
+    "tgk_cross_entropy": (i32, [vp, i32, i32, vp, vp, vp, vp, f32, i32]),
+    "tgk_sumsq_partials": (i32, [vp, vp, sz, vp, i32]),
+    "tgk_adamw": (i32, [vp, sz, vp, vp, vp, vp, vp, vp, i32, vp, vp, i32, f32, f32, f32, f32, f32, f32,
+                        C.c_uint64]),
+    "tgk_sample_batch": (i32, [vp, vp, i64, C.c_uint64, C.c_uint64, i32, i32, vp, vp]),
+    "tgk_position_means": (i32, [vp, vp, i32, i32, vp]),
 }
 ENGINE_ABI = {
     "tg_error": (C.c_char_p, []),

@@ -1,0 +1,588 @@
+// HBM-bound operators of the training step for gfx950: embedding, LayerNorm, cross-entropy,
+// AdamW on hi/lo split weights, batch sampling, loss bookkeeping.  Each stands in for a device
+// function of the reference named at its entry point.  All are single pass over their operands
+// with 16-byte accesses; reductions use a fixed order (no atomics), so results are reproducible.
+#include "common.h"
+#include "../../include/tgk_kernels.h"
+
+namespace {
+
+constexpr int MAX_LN_CHUNKS = 4; // 16-byte chunks per lane: rows up to 4*64*8 = 2048 columns
+
+TG_DEVICE void unpack8(const u32x4 &v, float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = bf16_lo(v[i]);
+        f[2 * i + 1] = bf16_hi(v[i]);
+    }
+}
+TG_DEVICE u32x4 pack8(const float (&f)[8]) {
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        v[i] = pack_bf16(f[2 * i], f[2 * i + 1]);
+    return v;
+}
+// fp32 master values of 8 consecutive parameters from their (hi, lo) halves (cuda/ops.cuh:6-9)
+TG_DEVICE void join8(const uint16_t *hi, const uint16_t *lo, float (&f)[8]) {
+    const u32x4 h = *reinterpret_cast<const u32x4 *>(hi), l = *reinterpret_cast<const u32x4 *>(lo);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __uint_as_float((h[i] << 16) | (l[i] & 0xffffu));
+        f[2 * i + 1] = __uint_as_float((h[i] & 0xffff0000u) | (l[i] >> 16));
+    }
+}
+TG_DEVICE uint64_t hash_u64(uint64_t x) { // utils.h:13-18
+    x += 0x9e3779b97f4a7c15ULL;
+    x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    x = (x ^ (x >> 27)) * 0x94d049bb133111ebULL;
+    return x ^ (x >> 31);
+}
+
+// ---- embedding ------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void embed_fwd_kernel(const uint8_t *__restrict__ x,
+                                                        const bf16_t *__restrict__ table,
+                                                        const bf16_t *__restrict__ positions,
+                                                        bf16_t *__restrict__ out, int rows, int T,
+                                                        int D) {
+    const int chunks = D >> 3;
+    const size_t total = size_t(rows) * chunks;
+    for (size_t i = blockIdx.x * size_t(256) + threadIdx.x; i < total; i += size_t(gridDim.x) * 256) {
+        const int row = int(i / chunks), c = int(i % chunks) * 8;
+        float a[8], b[8];
+        unpack8(*reinterpret_cast<const u32x4 *>(table + size_t(x[row]) * D + c), a);
+        unpack8(*reinterpret_cast<const u32x4 *>(positions + size_t(row % T) * D + c), b);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            a[k] += b[k];
+        *reinterpret_cast<u32x4 *>(out + size_t(row) * D + c) = pack8(a);
+    }
+}
+
+// dTable[v][c] = sum over tokens t with x[t] == v of dh[t][c], in token order.
+// grid (vocab, D/64); 256 threads = 4 token phases x 64 columns.
+__global__ __launch_bounds__(256) void embed_bwd_table_kernel(const uint8_t *__restrict__ x,
+                                                              const bf16_t *__restrict__ dh,
+                                                              float *__restrict__ dtable, int rows,
+                                                              int D, int accumulate) {
+    __shared__ uint8_t tokens[4096];
+    __shared__ float part[4][64];
+    const int v = blockIdx.x, col = blockIdx.y * 64 + (threadIdx.x & 63), phase = threadIdx.x >> 6;
+    float sum = 0.f;
+    for (int base = 0; base < rows; base += 4096) {
+        const int n = rows - base < 4096 ? rows - base : 4096;
+        __syncthreads();
+        for (int i = threadIdx.x; i < n; i += 256)
+            tokens[i] = x[base + i];
+        __syncthreads();
+        for (int i = phase; i < n; i += 4)
+            if (tokens[i] == v)
+                sum += bf16_to_float(dh[size_t(base + i) * D + col]);
+    }
+    part[phase][threadIdx.x & 63] = sum;
+    __syncthreads();
+    if (phase == 0) {
+        const int c = threadIdx.x;
+        float total = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
+        float *p = dtable + size_t(v) * D + col;
+        *p = accumulate ? *p + total : total;
+    }
+}
+// dPositions[p][c] = sum over sequences b of dh[b*T + p][c]
+__global__ __launch_bounds__(256) void embed_bwd_positions_kernel(const bf16_t *__restrict__ dh,
+                                                                  float *__restrict__ dpos, int B, int T,
+                                                                  int D, int accumulate) {
+    const size_t total = size_t(T) * D;
+    for (size_t i = blockIdx.x * size_t(256) + threadIdx.x; i < total; i += size_t(gridDim.x) * 256) {
+        float sum = 0.f;
+        for (int b = 0; b < B; ++b)
+            sum += bf16_to_float(dh[size_t(b) * total + i]);
+        dpos[i] = accumulate ? dpos[i] + sum : sum;
+    }
+}
+
+// ---- LayerNorm --------------------------------------------------------------------------------
+// One wave per row, the row lives in registers (two-pass mean / variance).
+__global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__restrict__ x,
+                                                            const uint16_t *__restrict__ gamma_hi,
+                                                            const uint16_t *__restrict__ gamma_lo,
+                                                            const uint16_t *__restrict__ beta_hi,
+                                                            const uint16_t *__restrict__ beta_lo,
+                                                            bf16_t *__restrict__ y, int rows, int D,
+                                                            float eps) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, chunks = D >> 3;
+    const float inv_d = 1.0f / D;
+    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+        float v[MAX_LN_CHUNKS][8];
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+            const int c = lane + j * 64;
+            if (c < chunks) {
+                unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    sum += v[j][k];
+            }
+        }
+        const float mean = wave_sum(sum) * inv_d;
+        float sq = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAX_LN_CHUNKS; ++j)
+            if (lane + j * 64 < chunks)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    v[j][k] -= mean;
+                    sq += v[j][k] * v[j][k];
+                }
+        const float inv = 1.0f / sqrtf(wave_sum(sq) * inv_d + eps);
+#pragma unroll
+        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+            const int c = lane + j * 64;
+            if (c < chunks) {
+                float gm[8], bt[8], o[8];
+                join8(gamma_hi + c * 8, gamma_lo + c * 8, gm);
+                join8(beta_hi + c * 8, beta_lo + c * 8, bt);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    o[k] = v[j][k] * inv * gm[k] + bt[k];
+                *reinterpret_cast<u32x4 *>(y + size_t(row) * D + c * 8) = pack8(o);
+            }
+        }
+    }
+}
+
+// dx (+ residual), and per-block partial sums of dgamma / dbeta into partial[block][2][D].
+__global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__restrict__ x,
+                                                            const bf16_t *__restrict__ dy,
+                                                            const uint16_t *__restrict__ gamma_hi,
+                                                            const uint16_t *__restrict__ gamma_lo,
+                                                            bf16_t *__restrict__ dx,
+                                                            float *__restrict__ partial, int rows, int D,
+                                                            float eps, int residual) {
+    extern __shared__ float lds[]; // [4 waves][2][D]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, chunks = D >> 3;
+    const float inv_d = 1.0f / D;
+    float dg[MAX_LN_CHUNKS][8], db[MAX_LN_CHUNKS][8], gm[MAX_LN_CHUNKS][8];
+#pragma unroll
+    for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+        const int c = lane + j * 64;
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            dg[j][k] = db[j][k] = gm[j][k] = 0.f;
+        if (c < chunks)
+            join8(gamma_hi + c * 8, gamma_lo + c * 8, gm[j]);
+    }
+    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+        float v[MAX_LN_CHUNKS][8], g[MAX_LN_CHUNKS][8];
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+            const int c = lane + j * 64;
+            if (c < chunks) {
+                unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
+                unpack8(*reinterpret_cast<const u32x4 *>(dy + size_t(row) * D + c * 8), g[j]);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    sum += v[j][k];
+            }
+        }
+        const float mean = wave_sum(sum) * inv_d;
+        float sq = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAX_LN_CHUNKS; ++j)
+            if (lane + j * 64 < chunks)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    v[j][k] -= mean;
+                    sq += v[j][k] * v[j][k];
+                }
+        const float inv = 1.0f / sqrtf(wave_sum(sq) * inv_d + eps);
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAX_LN_CHUNKS; ++j)
+            if (lane + j * 64 < chunks)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const float z = v[j][k] * inv, dz = g[j][k] * gm[j][k];
+                    v[j][k] = z;
+                    s1 += dz;
+                    s2 += dz * z;
+                    dg[j][k] += g[j][k] * z;
+                    db[j][k] += g[j][k];
+                }
+        s1 = wave_sum(s1) * inv_d;
+        s2 = wave_sum(s2) * inv_d;
+#pragma unroll
+        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+            const int c = lane + j * 64;
+            if (c < chunks) {
+                float o[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    o[k] = (g[j][k] * gm[j][k] - s1 - v[j][k] * s2) * inv;
+                bf16_t *p = dx + size_t(row) * D + c * 8;
+                if (residual) {
+                    // residual gradients stay in bf16 between operators (cuda/ops.cuh:74-76)
+                    float prior[8];
+                    unpack8(*reinterpret_cast<const u32x4 *>(p), prior);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        o[k] = prior[k] + round_bf16(o[k]);
+                }
+                *reinterpret_cast<u32x4 *>(p) = pack8(o);
+            }
+        }
+    }
+    float *mine = lds + wave * 2 * D;
+#pragma unroll
+    for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+        const int c = lane + j * 64;
+        if (c < chunks)
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                mine[c * 8 + k] = dg[j][k];
+                mine[D + c * 8 + k] = db[j][k];
+            }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 2 * D; i += 256)
+        partial[size_t(blockIdx.x) * 2 * D + i] =
+            (lds[i] + lds[2 * D + i]) + (lds[4 * D + i] + lds[6 * D + i]);
+}
+// dgamma[c] (+)= sum_b partial[b][0][c], dbeta likewise; fixed order over b
+__global__ __launch_bounds__(256) void layernorm_bwd_reduce_kernel(const float *__restrict__ partial,
+                                                                   int blocks, int D,
+                                                                   float *__restrict__ dgamma,
+                                                                   float *__restrict__ dbeta,
+                                                                   int accumulate) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= 2 * D)
+        return;
+    float sum = 0.f;
+    for (int b = 0; b < blocks; ++b)
+        sum += partial[size_t(b) * 2 * D + i];
+    float *out = i < D ? dgamma + i : dbeta + (i - D);
+    *out = accumulate ? *out + sum : sum;
+}
+
+// ---- cross-entropy over 256 byte classes ------------------------------------------------------
+// One wave per token: loss, optional fp32 copy of the logits, dlogits = RN((softmax - onehot) * k)
+// written in place over the bf16 logits (cuda/model.cuh:33-58).
+__global__ __launch_bounds__(256) void cross_entropy_kernel(bf16_t *__restrict__ logits,
+                                                            const uint8_t *__restrict__ y,
+                                                            float *__restrict__ loss,
+                                                            float *__restrict__ logits_f32, int rows,
+                                                            float inv_count, int write_grad) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+        bf16_t *p = logits + size_t(row) * 256 + lane * 4;
+        const u32x2 raw = *reinterpret_cast<const u32x2 *>(p);
+        float v[4] = {bf16_lo(raw.x), bf16_hi(raw.x), bf16_lo(raw.y), bf16_hi(raw.y)};
+        const float high = wave_max(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+        float e[4], sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            e[k] = __expf(v[k] - high);
+            sum += e[k];
+        }
+        sum = wave_sum(sum);
+        const int target = y[row];
+        const int t3 = target & 3;
+        const float own = t3 == 0 ? v[0] : t3 == 1 ? v[1] : t3 == 2 ? v[2] : v[3];
+        const float mine = (target >> 2) == lane ? own : 0.f;
+        const float picked = wave_sum(mine);
+        if (lane == 0)
+            loss[row] = high + __logf(sum) - picked;
+        if (logits_f32)
+            *reinterpret_cast<f32x4 *>(logits_f32 + size_t(row) * 256 + lane * 4) = f32x4{v[0], v[1], v[2], v[3]};
+        if (write_grad) {
+            const float inv = 1.0f / sum;
+            float gr[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                gr[k] = (e[k] * inv - (lane * 4 + k == target ? 1.f : 0.f)) * inv_count;
+            u32x2 out;
+            out.x = pack_bf16(gr[0], gr[1]);
+            out.y = pack_bf16(gr[2], gr[3]);
+            *reinterpret_cast<u32x2 *>(p) = out;
+        }
+    }
+}
+
+// ---- optimizer --------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void sumsq_kernel(const float *__restrict__ g, size_t n,
+                                                    float *__restrict__ partial) {
+    __shared__ float waves[4];
+    float sum = 0.f;
+    const size_t quads = n >> 2;
+    for (size_t i = blockIdx.x * size_t(256) + threadIdx.x; i < quads; i += size_t(gridDim.x) * 256) {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(g + i * 4);
+        sum += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+    if (blockIdx.x == 0 && threadIdx.x < int(n & 3)) {
+        const float v = g[(quads << 2) + threadIdx.x];
+        sum += v * v;
+    }
+    sum = wave_sum(sum);
+    if ((threadIdx.x & 63) == 0)
+        waves[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0)
+        partial[blockIdx.x] = (waves[0] + waves[1]) + (waves[2] + waves[3]);
+}
+
+struct AdamArgs {
+    float lr, beta1, beta2, eps, weight_decay, bc1, sqrt_bc2, clip;
+};
+// cuda/optim.cuh:67-106 on the (hi bf16, lo u16) weight halves (cuda/ops.cuh:6-14).
+// bounds: sorted starts of `segments` parameter ranges, bit 0 of flags[s] = weight decay.
+__global__ __launch_bounds__(256) void adamw_kernel(bf16_t *__restrict__ hi, uint16_t *__restrict__ lo,
+                                                    float *__restrict__ m, float *__restrict__ v,
+                                                    const float *__restrict__ g, size_t n,
+                                                    const float *__restrict__ norm_partials,
+                                                    int norm_count, const int64_t *__restrict__ bounds,
+                                                    const uint8_t *__restrict__ flags, int segments,
+                                                    AdamArgs a) {
+    __shared__ float waves[4];
+    __shared__ float clip_scale;
+    float scale = 1.f;
+    if (a.clip > 0.f) {
+        // every block folds the same partials in the same order (cuda/optim.cuh:67-80)
+        float sum = 0.f;
+        for (int i = threadIdx.x; i < norm_count; i += 256)
+            sum += norm_partials[i];
+        sum = wave_sum(sum);
+        if ((threadIdx.x & 63) == 0)
+            waves[threadIdx.x >> 6] = sum;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            clip_scale = fminf(1.f, a.clip / (sqrtf((waves[0] + waves[1]) + (waves[2] + waves[3])) + 1e-6f));
+        __syncthreads();
+        scale = clip_scale;
+    }
+    const size_t quads = n >> 2;
+    for (size_t q = blockIdx.x * size_t(256) + threadIdx.x; q < quads; q += size_t(gridDim.x) * 256) {
+        const size_t i = q * 4;
+        int lo_s = 0, hi_s = segments - 1; // last segment whose start <= i
+        while (lo_s < hi_s) {
+            const int mid = (lo_s + hi_s + 1) >> 1;
+            if (size_t(bounds[mid]) <= i)
+                lo_s = mid;
+            else
+                hi_s = mid - 1;
+        }
+        const float decay = (flags[lo_s] & 1) ? a.weight_decay : 0.f;
+        const f32x4 gv = *reinterpret_cast<const f32x4 *>(g + i);
+        f32x4 mv = *reinterpret_cast<const f32x4 *>(m + i), vv = *reinterpret_cast<const f32x4 *>(v + i);
+        const u32x2 hv = *reinterpret_cast<const u32x2 *>(hi + i), lv = *reinterpret_cast<const u32x2 *>(lo + i);
+        uint32_t bits[4] = {(hv.x << 16) | (lv.x & 0xffffu), (hv.x & 0xffff0000u) | (lv.x >> 16),
+                            (hv.y << 16) | (lv.y & 0xffffu), (hv.y & 0xffff0000u) | (lv.y >> 16)};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float gk = gv[k] * scale;
+            const float mk = mv[k] + (1.f - a.beta1) * (gk - mv[k]);
+            const float vk = a.beta2 * vv[k] + (1.f - a.beta2) * gk * gk;
+            mv[k] = mk;
+            vv[k] = vk;
+            const float w = __uint_as_float(bits[k]) * (1.f - a.lr * decay);
+            bits[k] = __float_as_uint(w - (a.lr / a.bc1) * mk / (sqrtf(vk) / a.sqrt_bc2 + a.eps));
+        }
+        *reinterpret_cast<f32x4 *>(m + i) = mv;
+        *reinterpret_cast<f32x4 *>(v + i) = vv;
+        u32x2 ho, lw;
+        ho.x = (bits[0] >> 16) | (bits[1] & 0xffff0000u);
+        ho.y = (bits[2] >> 16) | (bits[3] & 0xffff0000u);
+        lw.x = (bits[0] & 0xffffu) | (bits[1] << 16);
+        lw.y = (bits[2] & 0xffffu) | (bits[3] << 16);
+        *reinterpret_cast<u32x2 *>(hi + i) = ho;
+        *reinterpret_cast<u32x2 *>(lo + i) = lw;
+    }
+}
+
+// ---- data and loss bookkeeping ---------------------------------------------------------------
+// cuda/dataset.cuh:13-27; the window start is kept inside the data for contexts longer than 8
+__global__ __launch_bounds__(256) void sample_batch_kernel(const uint8_t *__restrict__ data, int64_t size,
+                                                           uint64_t seed, uint64_t step, int batch,
+                                                           int context, uint8_t *__restrict__ x,
+                                                           uint8_t *__restrict__ y) {
+    const int b = blockIdx.x;
+    const int64_t low = context > 8 ? context : 8;
+    const int64_t e = low + int64_t(hash_u64(seed + step * uint64_t(batch) + uint64_t(b)) % uint64_t(size - low));
+    for (int p = threadIdx.x; p < context; p += 256) {
+        x[size_t(b) * context + p] = data[e - context + p];
+        y[size_t(b) * context + p] = data[e - context + p + 1];
+    }
+}
+// cuda/trainer.cuh:79-100: mean over the batch per position, accumulated in double
+__global__ __launch_bounds__(256) void position_means_kernel(const float *__restrict__ token_loss,
+                                                             int batch, int context,
+                                                             float *__restrict__ out) {
+    const int p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= context)
+        return;
+    double sum = 0;
+    for (int b = 0; b < batch; ++b)
+        sum += token_loss[size_t(b) * context + p];
+    out[p] = float(sum / batch);
+}
+
+int grid_for(size_t work_items, int per_block, int cap = 4096) {
+    const size_t blocks = (work_items + per_block - 1) / per_block;
+    return int(blocks < size_t(cap) ? (blocks ? blocks : 1) : cap);
+}
+void aligned(const void *p, const char *name) {
+    if (!p || (reinterpret_cast<uintptr_t>(p) & 15))
+        throw std::invalid_argument(std::string(name) + " must be non-null and 16-byte aligned");
+}
+
+} // namespace
+
+extern "C" int tgk_embed_fwd(hipStream_t stream, int rows, int T, int D, const uint8_t *x,
+                             const uint16_t *table, const uint16_t *positions, uint16_t *out) {
+    return guarded([&] {
+        require(rows > 0 && T > 0 && D > 0 && D % 8 == 0, "embed_fwd: D must be a positive multiple of 8");
+        require(x != nullptr, "embed_fwd: missing tokens");
+        aligned(table, "embed_fwd: table");
+        aligned(positions, "embed_fwd: positions");
+        aligned(out, "embed_fwd: out");
+        hipLaunchKernelGGL(embed_fwd_kernel, dim3(grid_for(size_t(rows) * D / 8, 256)), dim3(256), 0, stream, x,
+                           table, positions, out, rows, T, D);
+        check_hip(hipGetLastError(), "embed_fwd launch: ");
+    });
+}
+
+extern "C" int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab, const uint8_t *x,
+                             const uint16_t *dh, float *dtable, float *dpositions, int accumulate) {
+    return guarded([&] {
+        require(B > 0 && T > 0 && D > 0 && D % 64 == 0, "embed_bwd: D must be a positive multiple of 64");
+        require(vocab > 0 && vocab <= 256, "embed_bwd: vocabulary is at most 256 (byte tokens)");
+        require(x && dh && dtable && dpositions, "embed_bwd: missing operand");
+        hipLaunchKernelGGL(embed_bwd_table_kernel, dim3(vocab, D / 64), dim3(256), 0, stream, x, dh, dtable,
+                           B * T, D, accumulate);
+        hipLaunchKernelGGL(embed_bwd_positions_kernel, dim3(grid_for(size_t(T) * D, 256)), dim3(256), 0, stream,
+                           dh, dpositions, B, T, D, accumulate);
+        check_hip(hipGetLastError(), "embed_bwd launch: ");
+    });
+}
+
+extern "C" int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint16_t *x,
+                                 const uint16_t *gamma_hi, const uint16_t *gamma_lo,
+                                 const uint16_t *beta_hi, const uint16_t *beta_lo, uint16_t *y, float eps) {
+    return guarded([&] {
+        require(rows > 0 && D > 0 && D % 8 == 0 && D <= MAX_LN_CHUNKS * 512,
+                "layernorm: D must be a multiple of 8, at most 2048");
+        aligned(x, "layernorm: x");
+        aligned(y, "layernorm: y");
+        aligned(gamma_hi, "layernorm: gamma_hi");
+        aligned(gamma_lo, "layernorm: gamma_lo");
+        aligned(beta_hi, "layernorm: beta_hi");
+        aligned(beta_lo, "layernorm: beta_lo");
+        hipLaunchKernelGGL(layernorm_fwd_kernel, dim3(grid_for(rows, 4, 8192)), dim3(256), 0, stream, x, gamma_hi,
+                           gamma_lo, beta_hi, beta_lo, y, rows, D, eps);
+        check_hip(hipGetLastError(), "layernorm_fwd launch: ");
+    });
+}
+
+static int layernorm_bwd_blocks(int rows) {
+    return grid_for(rows, 16, 1024);
+}
+extern "C" size_t tgk_layernorm_bwd_workspace(int rows, int D) {
+    return rows > 0 && D > 0 ? size_t(layernorm_bwd_blocks(rows)) * 2 * D * sizeof(float) : 0;
+}
+extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint16_t *x,
+                                 const uint16_t *dy, const uint16_t *gamma_hi, const uint16_t *gamma_lo,
+                                 uint16_t *dx, float *dgamma, float *dbeta, float eps, int residual,
+                                 int accumulate, void *workspace, size_t workspace_bytes) {
+    return guarded([&] {
+        require(rows > 0 && D > 0 && D % 8 == 0 && D <= MAX_LN_CHUNKS * 512,
+                "layernorm: D must be a multiple of 8, at most 2048");
+        aligned(x, "layernorm: x");
+        aligned(dy, "layernorm: dy");
+        aligned(dx, "layernorm: dx");
+        aligned(gamma_hi, "layernorm: gamma_hi");
+        aligned(gamma_lo, "layernorm: gamma_lo");
+        require(dgamma && dbeta, "layernorm_bwd: missing operand");
+        require(workspace && workspace_bytes >= tgk_layernorm_bwd_workspace(rows, D),
+                "layernorm_bwd: workspace too small (see tgk_layernorm_bwd_workspace)");
+        const int blocks = layernorm_bwd_blocks(rows);
+        float *partial = static_cast<float *>(workspace);
+        hipLaunchKernelGGL(layernorm_bwd_kernel, dim3(blocks), dim3(256), size_t(8) * D * sizeof(float), stream, x,
+                           dy, gamma_hi, gamma_lo, dx, partial, rows, D, eps, residual);
+        hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3((2 * D + 255) / 256), dim3(256), 0, stream, partial,
+                           blocks, D, dgamma, dbeta, accumulate);
+        check_hip(hipGetLastError(), "layernorm_bwd launch: ");
+    });
+}
+
+extern "C" int tgk_cross_entropy(hipStream_t stream, int rows, int vocab, uint16_t *logits,
+                                 const uint8_t *y, float *loss, float *logits_f32, float inv_count,
+                                 int write_grad) {
+    return guarded([&] {
+        require(rows > 0, "cross_entropy: empty batch");
+        require(vocab == 256, "cross_entropy: vocabulary must be 256 (byte tokens)");
+        aligned(logits, "cross_entropy: logits");
+        require(y && loss, "cross_entropy: missing operand");
+        require(!logits_f32 || !(reinterpret_cast<uintptr_t>(logits_f32) & 15),
+                "cross_entropy: fp32 logits must be 16-byte aligned");
+        hipLaunchKernelGGL(cross_entropy_kernel, dim3(grid_for(rows, 4, 8192)), dim3(256), 0, stream, logits, y,
+                           loss, logits_f32, rows, inv_count, write_grad);
+        check_hip(hipGetLastError(), "cross_entropy launch: ");
+    });
+}
+
+extern "C" int tgk_sumsq_partials(hipStream_t stream, const float *g, size_t n, float *partials,
+                                  int count) {
+    return guarded([&] {
+        aligned(g, "sumsq: g");
+        require(partials && count > 0 && count <= 4096, "sumsq: 1..4096 partials");
+        hipLaunchKernelGGL(sumsq_kernel, dim3(count), dim3(256), 0, stream, g, n, partials);
+        check_hip(hipGetLastError(), "sumsq launch: ");
+    });
+}
+
+extern "C" int tgk_adamw(hipStream_t stream, size_t n, uint16_t *weight_hi, uint16_t *weight_lo, float *m,
+                         float *v, const float *g, const float *norm_partials, int norm_count,
+                         const int64_t *segment_starts, const uint8_t *segment_flags, int segments,
+                         float lr, float beta1, float beta2, float eps, float weight_decay, float clip,
+                         uint64_t step) {
+    return guarded([&] {
+        require(n > 0 && n % 4 == 0, "adamw: parameter count must be a positive multiple of 4");
+        aligned(weight_hi, "adamw: weight_hi");
+        aligned(weight_lo, "adamw: weight_lo");
+        aligned(m, "adamw: m");
+        aligned(v, "adamw: v");
+        aligned(g, "adamw: g");
+        require(segment_starts && segment_flags && segments > 0, "adamw: missing segment table");
+        require(!(clip > 0.f) || (norm_partials && norm_count > 0), "adamw: clipping needs the norm partials");
+        // bias correction with the current beta1 (cuda/optim.cuh:90-91), evaluated on the host in fp32
+        AdamArgs a{lr, beta1, beta2, eps, weight_decay, 1.f - powf(beta1, float(step + 1)),
+                   sqrtf(1.f - powf(beta2, float(step + 1))), clip};
+        hipLaunchKernelGGL(adamw_kernel, dim3(grid_for(n / 4, 256, 8192)), dim3(256), 0, stream, weight_hi,
+                           weight_lo, m, v, g, n, norm_partials, norm_count, segment_starts, segment_flags,
+                           segments, a);
+        check_hip(hipGetLastError(), "adamw launch: ");
+    });
+}
+
+extern "C" int tgk_sample_batch(hipStream_t stream, const uint8_t *data, int64_t size, uint64_t seed,
+                                uint64_t step, int batch, int context, uint8_t *x, uint8_t *y) {
+    return guarded([&] {
+        require(data && x && y, "sample_batch: missing operand");
+        require(batch > 0 && context > 0, "sample_batch: empty batch");
+        require(size > (context > 8 ? context : 8), "sample_batch: dataset shorter than one window");
+        hipLaunchKernelGGL(sample_batch_kernel, dim3(batch), dim3(256), 0, stream, data, size, seed, step, batch,
+                           context, x, y);
+        check_hip(hipGetLastError(), "sample_batch launch: ");
+    });
+}
+
+extern "C" int tgk_position_means(hipStream_t stream, const float *token_loss, int batch, int context,
+                                  float *out) {
+    return guarded([&] {
+        require(token_loss && out && batch > 0 && context > 0, "position_means: missing operand");
+        hipLaunchKernelGGL(position_means_kernel, dim3((context + 255) / 256), dim3(256), 0, stream, token_loss,
+                           batch, context, out);
+        check_hip(hipGetLastError(), "position_means launch: ");
+    });
+}
