@@ -79,8 +79,8 @@ def test_onecycle_matches_torch_scheduler(orc, total):
 def test_onecycle_matches_reference_header(orc):
     if orc.ref_host() is None:
         pytest.skip("oracle/_ref not built (reference tree absent)")
-    for total in (8, 20, 37, 48829):
-        for step in sorted(set([0, 1, total // 3, total // 2, total - 1])):
+    for total in (1, 8, 20, 37, 48829):
+        for step in sorted(set([0, min(1, total - 1), total // 3, total // 2, total - 1])):
             assert orc.onecycle_point(total, step) == orc.onecycle_point(total, step, use_ref=True)
     with pytest.raises(ValueError):
         orc.onecycle_point(20, 25, use_ref=True)

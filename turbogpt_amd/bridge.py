@@ -36,8 +36,72 @@ KERNEL_ABI = {
     "tgk_sample_batch": (i32, [vp, vp, i64, C.c_uint64, C.c_uint64, i32, i32, vp, vp]),
     "tgk_position_means": (i32, [vp, vp, i32, i32, vp]),
 }
+u64 = C.c_uint64
+
+
+class Config(C.Structure):
+    """config.h:5-13 of the reference; same field order and defaults as tests/bridge.py:7-15."""
+    _fields_ = [(x, C.c_int) for x in ("depth", "context", "batch", "device", "blocks", "ns_steps")] + [
+        (x, C.c_float) for x in ("learning_rate", "muon_lr", "beta1", "beta2", "momentum", "weight_decay",
+                                 "epsilon", "clip")] + [("seed", C.c_uint64), ("inflight", C.c_int)]
+
+    def __init__(self, **kwargs):
+        super().__init__(4, 4, 16, 0, 0, 5, .0006, .02, .9, .95, .95, .1, 1e-8, 1., 3407, 1)
+        for key, value in kwargs.items():
+            setattr(self, key, value)
+
+
+class ModelConfig(C.Structure):
+    """TgModelConfig of include/tg_runtime.h: the reference Config plus the model shape."""
+    _fields_ = [("base", Config), ("d_model", C.c_int), ("heads", C.c_int), ("vocab", C.c_int), ("ffn", C.c_int),
+                ("ln_eps", C.c_float), ("reserved", C.c_int * 3)]
+
+    def __init__(self, d_model=768, heads=None, ffn=None, vocab=256, ln_eps=1e-5, **base):
+        super().__init__()
+        self.base = Config(**base)
+        self.d_model, self.heads = d_model, heads if heads is not None else d_model // 64
+        self.vocab, self.ffn, self.ln_eps = vocab, ffn if ffn is not None else 4 * d_model, ln_eps
+
+
+class OneCycle(C.Structure):
+    """optim.h:6-13."""
+    _fields_ = [("total_steps", C.c_int)] + [
+        (name, C.c_double) for name in ("warmup_fraction", "initial_lr_fraction", "final_lr_fraction",
+                                        "low_momentum", "high_momentum")]
+
+    def __init__(self, total_steps):
+        super().__init__(total_steps, .3, .04, .000004, .85, .95)
+
+
+class StepRates(C.Structure):
+    _fields_ = [("multiplier", C.c_float), ("momentum", C.c_float)]
+
+
+# every symbol include/tg_runtime.h declares
 ENGINE_ABI = {
     "tg_error": (C.c_char_p, []),
+    "tg_create": (vp, [C.POINTER(Config)]),
+    "tg_create_ex": (vp, [C.POINTER(ModelConfig)]),
+    "tg_destroy": (None, [vp]),
+    "tg_parameter_count": (i32, [vp]),
+    "tg_blocks": (i32, [vp]),
+    "tg_shared_bytes": (i32, [vp]),
+    "tg_set_weights": (i32, [vp, vp]),
+    "tg_get_weights": (i32, [vp, vp]),
+    "tg_get_optimizer_state": (i32, [vp, vp, vp, C.POINTER(u64)]),
+    "tg_set_optimizer_state": (i32, [vp, vp, vp, u64]),
+    "tg_memory": (i32, [vp, C.POINTER(C.c_double)]),
+    "tg_set_data": (i32, [vp, vp, i64]),
+    "tg_train": (i32, [vp, i32]),
+    "tg_get_training_losses": (i32, [vp, vp, i32]),
+    "tg_training_versions": (i32, [vp, vp, i32]),
+    "tg_pipeline_stats": (i32, [vp, C.POINTER(C.c_double), C.POINTER(i32)]),
+    "tg_onecycle_point": (i32, [C.POINTER(OneCycle), i32, C.POINTER(StepRates)]),
+    "tg_set_onecycle": (i32, [vp, C.POINTER(OneCycle)]),
+    "tg_batch": (i32, [vp] * 6),
+    "tg_predict": (i32, [vp, vp, vp]),
+    "tg_optimizer_test": (i32, [vp, vp, i32]),
+    "tg_synchronize": (i32, [vp]),
 }
 
 
@@ -65,3 +129,96 @@ def check(status):
     if status < 0:
         raise RuntimeError(library().tg_error().decode())
     return status
+
+
+class Native:
+    """One engine, as in tests/bridge.py:29-81 of the reference, over tg_create_ex."""
+
+    def __init__(self, config):
+        import numpy as np
+        self.np = np
+        self.config = config
+        self.lib = library()
+        self.handle = self.lib.tg_create_ex(C.byref(config))
+        if not self.handle:
+            raise RuntimeError(self.lib.tg_error().decode())
+        self.count = self.lib.tg_parameter_count(self.handle)
+
+    def check(self, value):
+        if value < 0:
+            raise RuntimeError(self.lib.tg_error().decode())
+
+    def close(self):
+        if self.handle:
+            self.lib.tg_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def set_weights(self, w):
+        w = self.np.ascontiguousarray(w, dtype=self.np.float32)
+        assert w.size == self.count
+        self.check(self.lib.tg_set_weights(self.handle, w.ctypes.data))
+
+    def weights(self):
+        w = self.np.empty(self.count, self.np.float32)
+        self.check(self.lib.tg_get_weights(self.handle, w.ctypes.data))
+        return w
+
+    def optimizer_state(self):
+        m, v = self.np.empty(self.count, self.np.float32), self.np.empty(self.count, self.np.float32)
+        step = u64()
+        self.check(self.lib.tg_get_optimizer_state(self.handle, m.ctypes.data, v.ctypes.data, C.byref(step)))
+        return m, v, step.value
+
+    def set_optimizer_state(self, m, v, step):
+        m = self.np.ascontiguousarray(m, dtype=self.np.float32)
+        v = self.np.ascontiguousarray(v, dtype=self.np.float32)
+        self.check(self.lib.tg_set_optimizer_state(self.handle, m.ctypes.data, v.ctypes.data, step))
+
+    def set_data(self, data):
+        data = self.np.ascontiguousarray(data, dtype=self.np.uint8)
+        self.check(self.lib.tg_set_data(self.handle, data.ctypes.data, data.size))
+
+    def set_onecycle(self, total_steps):
+        self.check(self.lib.tg_set_onecycle(self.handle, C.byref(OneCycle(total_steps))))
+
+    def train(self, steps):
+        self.check(self.lib.tg_train(self.handle, steps))
+
+    def training_losses(self, count):
+        out = self.np.empty((count, self.config.base.context), self.np.float32)
+        self.check(self.lib.tg_get_training_losses(self.handle, out.ctypes.data, count))
+        return out
+
+    def optimizer_test(self, grad, steps=1):
+        grad = self.np.ascontiguousarray(grad, dtype=self.np.float32)
+        assert grad.size == self.count
+        self.check(self.lib.tg_optimizer_test(self.handle, grad.ctypes.data, steps))
+
+    def synchronize(self):
+        self.check(self.lib.tg_synchronize(self.handle))
+
+    def batch(self, x, y, backward=True):
+        np = self.np
+        base = self.config.base
+        x, y = np.ascontiguousarray(x, dtype=np.uint8), np.ascontiguousarray(y, dtype=np.uint8)
+        assert x.shape == y.shape == (base.batch, base.context)
+        logits = np.empty((*x.shape, self.config.vocab), np.float32)
+        grad = np.empty(self.count, np.float32) if backward else None
+        losses = np.empty(base.context, np.float32)
+        self.check(self.lib.tg_batch(self.handle, x.ctypes.data, y.ctypes.data, logits.ctypes.data,
+                                     grad.ctypes.data if grad is not None else None, losses.ctypes.data))
+        return logits, grad, losses
+
+    def predict(self, context):
+        np = self.np
+        context = np.ascontiguousarray(context, dtype=np.uint8)
+        assert context.size == self.config.base.context
+        logits = np.empty(self.config.vocab, np.float32)
+        self.check(self.lib.tg_predict(self.handle, context.ctypes.data, logits.ctypes.data))
+        return logits

@@ -1,0 +1,582 @@
+// Engine behind the tg_* C ABI: owns every device buffer, and runs the training step as a
+// sequence of kernel launches on one HIP stream.  Host-side counterpart of the reference's
+// cuda/runtime.cu + cuda/engine_state.cu (resource ownership, transfers, entry points) and of the
+// op sequencing that its persistent kernel does on the device (cuda/trainer.cuh:103-125,
+// cuda/model.cuh:8-99).  All arithmetic is in the tgk_* kernels; this file only sequences them.
+#include "common.h"
+#include "../../include/tg_model.h"
+#include "../../include/tgk_kernels.h"
+#include <algorithm>
+#include <climits>
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+namespace {
+
+constexpr int MaxLaunchSteps = 4096; // cuda/types.cuh:10
+constexpr int NormPartials = 1024;
+
+struct LayerBuffers {
+    bf16_t *n1, *qkv, *o, *mid, *n2, *u, *a;
+    float *lse;
+};
+
+void ok(int status) {
+    if (status < 0)
+        throw std::runtime_error(tg_last_error);
+}
+
+// optim.h:18-44
+StepRates onecycle_point(const OneCycle &s, int step) {
+    if (s.total_steps < 1 || step < 0 || step >= s.total_steps ||
+        !(s.warmup_fraction > 0 && s.warmup_fraction < 1) ||
+        !(s.initial_lr_fraction > 0 && s.initial_lr_fraction < 1) ||
+        !(s.final_lr_fraction > 0 && s.final_lr_fraction <= s.initial_lr_fraction) ||
+        !(s.low_momentum >= 0 && s.low_momentum < 1) ||
+        !(s.high_momentum >= s.low_momentum && s.high_momentum < 1))
+        throw std::runtime_error("Invalid OneCycle schedule or step");
+    const double warmup_steps = s.warmup_fraction * s.total_steps - 1;
+    if (warmup_steps == 0)
+        throw std::runtime_error("OneCycle warmup must span at least two steps");
+    const bool warming = step <= warmup_steps;
+    const double fraction =
+        warming ? step / warmup_steps : (step - warmup_steps) / (s.total_steps - 1 - warmup_steps);
+    const double c = 0.5 * (1 + std::cos(3.14159265358979323846 * fraction));
+    const auto between = [c](double from, double to) { return to + (from - to) * c; };
+    return {float(warming ? between(s.initial_lr_fraction, 1.0) : between(1.0, s.final_lr_fraction)),
+            float(warming ? between(s.high_momentum, s.low_momentum)
+                          : between(s.low_momentum, s.high_momentum))};
+}
+
+} // namespace
+
+struct Engine {
+    TgModelConfig config{};
+    TgParameterLayout layout{};
+    hipStream_t stream = nullptr;
+    std::vector<void *> allocations;
+    size_t allocated_bytes = 0;
+    int compute_units = 0;
+
+    uint16_t *weight_hi = nullptr, *weight_lo = nullptr;
+    float *momentum = nullptr, *variance = nullptr, *gradient = nullptr;
+    float *norm_partials = nullptr, *token_losses = nullptr, *loss_history = nullptr;
+    int64_t *segment_starts = nullptr;
+    uint8_t *segment_flags = nullptr;
+    int segments = 0;
+    uint8_t *data = nullptr, *input = nullptr, *target = nullptr;
+    int64_t data_size = 0;
+
+    std::vector<bf16_t *> x; // x[l] = input of block l; x[depth] = output of the last block
+    std::vector<LayerBuffers> layers;
+    bf16_t *nf = nullptr, *logits = nullptr, *dh = nullptr, *t1 = nullptr, *du = nullptr, *dqkv = nullptr;
+    float *logits_f32 = nullptr;
+    void *workspace = nullptr;
+    size_t workspace_bytes = 0;
+
+    std::vector<StepRates> schedule;
+    uint64_t step = 0;
+    int last_train_steps = 0;
+
+    int tokens() const { return config.base.batch * config.base.context; }
+
+    template <class T> void allocate(T *&ptr, size_t n, bool zero = true) { // cuda/engine_internal.h:17-27
+        void *raw = nullptr;
+        check_hip(hipMalloc(&raw, n * sizeof(T)), "allocation: ");
+        ptr = static_cast<T *>(raw);
+        allocations.push_back(raw);
+        allocated_bytes += n * sizeof(T);
+        if (zero)
+            check_hip(hipMemsetAsync(raw, 0, n * sizeof(T), stream));
+    }
+    void use_device() const { check_hip(hipSetDevice(config.base.device)); }
+    void sync() const { check_hip(hipStreamSynchronize(stream)); }
+    template <class T> void upload(T *device, const T *host, size_t n) {
+        check_hip(hipMemcpyAsync(device, host, n * sizeof(T), hipMemcpyHostToDevice, stream));
+    }
+    template <class T> void download(T *host, const T *device, size_t n) {
+        check_hip(hipMemcpyAsync(host, device, n * sizeof(T), hipMemcpyDeviceToHost, stream));
+    }
+    ~Engine() { // cuda/engine_internal.h:28-37
+        (void)hipSetDevice(config.base.device);
+        if (stream)
+            (void)hipStreamSynchronize(stream);
+        for (void *allocation : allocations)
+            (void)hipFree(allocation);
+        if (stream)
+            (void)hipStreamDestroy(stream);
+    }
+
+    const uint16_t *w(int64_t offset) const { return weight_hi + offset; }
+    const uint16_t *wl(int64_t offset) const { return weight_lo + offset; }
+
+    // cuda/model.cuh:8-59.  evaluate: logits stay logits; otherwise they are replaced by dlogits.
+    void forward(const uint8_t *tokens_in, const uint8_t *targets, bool with_gradient, float *logits_out) {
+        const Config &c = config.base;
+        const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
+        const float scale = 1.0f / std::sqrt(float(d / config.heads));
+        ok(tgk_embed_fwd(stream, M, T, d, tokens_in, w(layout.embedding), w(layout.positions), x[0]));
+        for (int l = 0; l < c.depth; ++l) {
+            const TgLayerParameters &p = layout.layers[l];
+            LayerBuffers &b = layers[l];
+            ok(tgk_layernorm_fwd(stream, M, d, x[l], w(p.ln1_g), wl(p.ln1_g), w(p.ln1_b), wl(p.ln1_b), b.n1,
+                                 config.ln_eps));
+            ok(tgk_gemm_fwd(stream, M, 3 * d, d, b.n1, d, w(p.qkv), d, b.qkv, 3 * d, nullptr, 0, nullptr, 0));
+            ok(tgk_attn_fwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
+                            3 * d, b.o, d, b.lse, scale));
+            ok(tgk_gemm_fwd(stream, M, d, d, b.o, d, w(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
+            ok(tgk_layernorm_fwd(stream, M, d, b.mid, w(p.ln2_g), wl(p.ln2_g), w(p.ln2_b), wl(p.ln2_b), b.n2,
+                                 config.ln_eps));
+            ok(tgk_gemm_fwd(stream, M, F, d, b.n2, d, w(p.mlp_up), d, b.u, F, nullptr, 0, b.a, F));
+            ok(tgk_gemm_fwd(stream, M, d, F, b.a, F, w(p.mlp_down), F, x[l + 1], d, b.mid, d, nullptr, 0));
+        }
+        ok(tgk_layernorm_fwd(stream, M, d, x[c.depth], w(layout.lnf_g), wl(layout.lnf_g), w(layout.lnf_b),
+                             wl(layout.lnf_b), nf, config.ln_eps));
+        ok(tgk_gemm_fwd(stream, M, V, d, nf, d, w(layout.head), d, logits, V, nullptr, 0, nullptr, 0));
+        ok(tgk_cross_entropy(stream, M, V, logits, targets, token_losses, logits_out, 1.0f / float(M),
+                             with_gradient ? 1 : 0));
+    }
+
+    // cuda/model.cuh:61-99.  Every element of `gradient` is overwritten: nothing needs zeroing.
+    void backward(const uint8_t *tokens_in) {
+        const Config &c = config.base;
+        const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
+        const float scale = 1.0f / std::sqrt(float(d / config.heads));
+        float *g = gradient;
+        ok(tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
+        ok(tgk_gemm_dgrad(stream, M, V, d, logits, V, w(layout.head), d, t1, d, nullptr, 0));
+        ok(tgk_layernorm_bwd(stream, M, d, x[c.depth], t1, w(layout.lnf_g), wl(layout.lnf_g), dh,
+                             g + layout.lnf_g, g + layout.lnf_b, config.ln_eps, 0, 0, workspace, workspace_bytes));
+        for (int l = c.depth - 1; l >= 0; --l) {
+            const TgLayerParameters &p = layout.layers[l];
+            LayerBuffers &b = layers[l];
+            ok(tgk_gemm_wgrad(stream, M, d, F, dh, d, b.a, F, g + p.mlp_down, F, 0, workspace, workspace_bytes));
+            ok(tgk_gemm_dgrad(stream, M, d, F, dh, d, w(p.mlp_down), F, du, F, b.u, F));
+            ok(tgk_gemm_wgrad(stream, M, F, d, du, F, b.n2, d, g + p.mlp_up, d, 0, workspace, workspace_bytes));
+            ok(tgk_gemm_dgrad(stream, M, F, d, du, F, w(p.mlp_up), d, t1, d, nullptr, 0));
+            ok(tgk_layernorm_bwd(stream, M, d, b.mid, t1, w(p.ln2_g), wl(p.ln2_g), dh, g + p.ln2_g, g + p.ln2_b,
+                                 config.ln_eps, 1, 0, workspace, workspace_bytes));
+            ok(tgk_gemm_wgrad(stream, M, d, d, dh, d, b.o, d, g + p.attn_out, d, 0, workspace, workspace_bytes));
+            ok(tgk_gemm_dgrad(stream, M, d, d, dh, d, w(p.attn_out), d, t1, d, nullptr, 0));
+            ok(tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
+                            3 * d, b.o, d, b.lse, t1, d, dqkv, dqkv + d, dqkv + 2 * d, 3 * d, scale, workspace,
+                            workspace_bytes));
+            ok(tgk_gemm_wgrad(stream, M, 3 * d, d, dqkv, 3 * d, b.n1, d, g + p.qkv, d, 0, workspace,
+                              workspace_bytes));
+            ok(tgk_gemm_dgrad(stream, M, 3 * d, d, dqkv, 3 * d, w(p.qkv), d, t1, d, nullptr, 0));
+            ok(tgk_layernorm_bwd(stream, M, d, x[l], t1, w(p.ln1_g), wl(p.ln1_g), dh, g + p.ln1_g, g + p.ln1_b,
+                                 config.ln_eps, 1, 0, workspace, workspace_bytes));
+        }
+        ok(tgk_embed_bwd(stream, c.batch, T, d, V, tokens_in, dh, g + layout.embedding, g + layout.positions, 0));
+    }
+
+    // cuda/optim.cuh:66-106 for optimizer step `at` (0-based)
+    void optimize(uint64_t at) {
+        const Config &c = config.base;
+        float lr = c.learning_rate, beta1 = c.beta1;
+        if (!schedule.empty()) {
+            lr *= schedule[at].multiplier;
+            beta1 = schedule[at].momentum;
+        }
+        if (c.clip > 0)
+            ok(tgk_sumsq_partials(stream, gradient, size_t(layout.count), norm_partials, NormPartials));
+        ok(tgk_adamw(stream, size_t(layout.count), weight_hi, weight_lo, momentum, variance, gradient,
+                     norm_partials, NormPartials, segment_starts, segment_flags, segments, lr, beta1, c.beta2,
+                     c.epsilon, c.weight_decay, c.clip, at));
+    }
+
+    void read_losses(float *out) { // cuda/runtime.cu:279-290
+        const Config &c = config.base;
+        std::vector<float> losses(static_cast<size_t>(tokens()));
+        download(losses.data(), token_losses, losses.size());
+        sync();
+        for (int p = 0; p < c.context; ++p) {
+            double sum = 0;
+            for (int b = 0; b < c.batch; ++b)
+                sum += losses[size_t(b) * c.context + p];
+            out[p] = float(sum / c.batch);
+        }
+    }
+};
+
+namespace {
+
+void validate(const TgModelConfig &m) {
+    const Config &c = m.base;
+    if (c.depth < 1 || c.depth > TG_MAX_DEPTH)
+        throw std::runtime_error("Supported: depth 1..64");
+    if (m.vocab != 256)
+        throw std::runtime_error("Supported: vocabulary 256 (byte tokens)");
+    if (m.d_model < 128 || m.d_model % 128 || m.d_model > 2048)
+        throw std::runtime_error("Supported: d_model a multiple of 128, at most 2048");
+    if (m.heads * 64 != m.d_model)
+        throw std::runtime_error("Supported: head_dim 64 (heads = d_model / 64)");
+    if (m.ffn < 128 || m.ffn % 128)
+        throw std::runtime_error("Supported: ffn a multiple of 128");
+    if (c.context < 128 || c.context % 128)
+        throw std::runtime_error("Supported: context a multiple of 128");
+    if (c.batch < 1 || int64_t(c.batch) * c.context > (int64_t(1) << 24))
+        throw std::runtime_error("Supported: batch >= 1 with batch*context <= 2^24 tokens");
+    if (c.inflight != 1)
+        throw std::runtime_error("inflight must be 1: the stale-gradient pipeline is not built");
+    if (!(m.ln_eps > 0))
+        throw std::runtime_error("ln_eps must be positive");
+}
+
+void build_segments(Engine *e) {
+    // weight-decay groups: block matrices and head decay, everything else does not
+    std::vector<int64_t> starts;
+    std::vector<uint8_t> flags;
+    const auto add = [&](int64_t start, bool decay) {
+        if (!flags.empty() && flags.back() == uint8_t(decay))
+            return;
+        starts.push_back(start);
+        flags.push_back(uint8_t(decay));
+    };
+    const TgParameterLayout &p = e->layout;
+    add(p.embedding, false);
+    for (int l = 0; l < e->config.base.depth; ++l) {
+        const TgLayerParameters &b = p.layers[l];
+        add(b.ln1_g, false);
+        add(b.qkv, true);
+        add(b.ln2_g, false);
+        add(b.mlp_up, true);
+    }
+    add(p.lnf_g, false);
+    add(p.head, true);
+    e->segments = int(starts.size());
+    e->allocate(e->segment_starts, starts.size(), false);
+    e->allocate(e->segment_flags, flags.size(), false);
+    e->upload(e->segment_starts, starts.data(), starts.size());
+    e->upload(e->segment_flags, flags.data(), flags.size());
+    e->sync(); // the host vectors go out of scope
+}
+
+} // namespace
+
+TG_API Engine *tg_create(const Config *) {
+    tg_last_error = "tg_create builds the reference's fixed width-16 network, which this library does not "
+                    "contain; describe the model with TgModelConfig and call tg_create_ex";
+    return nullptr;
+}
+
+TG_API Engine *tg_create_ex(const TgModelConfig *model) {
+    Engine *e = nullptr;
+    try {
+        if (!model)
+            throw std::runtime_error("Missing configuration");
+        validate(*model);
+        int devices = 0;
+        check_hip(hipGetDeviceCount(&devices), "device query: ");
+        if (model->base.device < 0 || model->base.device >= devices)
+            throw std::runtime_error("No such device");
+        check_hip(hipSetDevice(model->base.device));
+        hipDeviceProp_t prop{};
+        check_hip(hipGetDeviceProperties(&prop, model->base.device));
+        if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            throw std::runtime_error(std::string("Requires an MI355X-class device (gfx950), found ") +
+                                     prop.gcnArchName);
+        e = new Engine;
+        e->config = *model;
+        e->layout = tg_parameter_layout(model);
+        e->compute_units = prop.multiProcessorCount;
+        if (e->layout.count > INT_MAX)
+            throw std::runtime_error("Parameter count exceeds signed 32-bit indexing");
+        check_hip(hipStreamCreate(&e->stream));
+
+        const Config &c = model->base;
+        const size_t P = size_t(e->layout.count), M = size_t(e->tokens()), d = size_t(model->d_model);
+        const size_t F = size_t(model->ffn), V = size_t(model->vocab);
+        e->allocate(e->weight_hi, P);
+        e->allocate(e->weight_lo, P);
+        e->allocate(e->momentum, P);
+        e->allocate(e->variance, P);
+        e->allocate(e->gradient, P);
+        e->allocate(e->norm_partials, NormPartials);
+        e->allocate(e->token_losses, M);
+        e->allocate(e->loss_history, size_t(MaxLaunchSteps) * c.context);
+        e->allocate(e->input, M);
+        e->allocate(e->target, M);
+        build_segments(e);
+        e->x.resize(c.depth + 1);
+        e->layers.resize(c.depth);
+        for (int l = 0; l <= c.depth; ++l)
+            e->allocate(e->x[l], M * d, false);
+        for (int l = 0; l < c.depth; ++l) {
+            LayerBuffers &b = e->layers[l];
+            e->allocate(b.n1, M * d, false);
+            e->allocate(b.qkv, M * 3 * d, false);
+            e->allocate(b.o, M * d, false);
+            e->allocate(b.lse, size_t(c.batch) * model->heads * c.context, false);
+            e->allocate(b.mid, M * d, false);
+            e->allocate(b.n2, M * d, false);
+            e->allocate(b.u, M * F, false);
+            e->allocate(b.a, M * F, false);
+        }
+        e->allocate(e->nf, M * d, false);
+        e->allocate(e->logits, M * V, false);
+        e->allocate(e->dh, M * d, false);
+        e->allocate(e->t1, M * d, false);
+        e->allocate(e->du, M * F, false);
+        e->allocate(e->dqkv, M * 3 * d, false);
+        size_t need = tgk_attn_bwd_workspace(c.batch, model->heads, c.context);
+        need = std::max(need, tgk_layernorm_bwd_workspace(int(M), int(d)));
+        need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(V), int(d)));
+        need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(d), int(F)));
+        need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(F), int(d)));
+        need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(d), int(d)));
+        need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(3 * d), int(d)));
+        e->workspace_bytes = need;
+        uint8_t *ws = nullptr;
+        e->allocate(ws, need, false);
+        e->workspace = ws;
+        e->sync();
+        return e;
+    } catch (const std::exception &error) {
+        tg_last_error = error.what();
+        delete e;
+        return nullptr;
+    }
+}
+
+TG_API void tg_destroy(Engine *e) {
+    delete e;
+}
+TG_API int tg_parameter_count(Engine *e) {
+    return int(e->layout.count);
+}
+TG_API int tg_blocks(Engine *e) {
+    return e->compute_units;
+}
+TG_API int tg_shared_bytes(Engine *) {
+    return 2 * (256 + 256) * 72 * 2; // the 256x256 GEMM tile: two stages of (256+256) rows x 72 bf16
+}
+TG_API int tg_synchronize(Engine *e) {
+    return guarded([&] {
+        e->use_device();
+        e->sync();
+    });
+}
+TG_API int tg_memory(Engine *e, double *used_gb) {
+    return guarded([&] {
+        if (!used_gb)
+            throw std::runtime_error("Missing memory output");
+        *used_gb = double(e->allocated_bytes) / (1024.0 * 1024.0 * 1024.0);
+    });
+}
+
+// cuda/engine_state.cu:7-35
+TG_API int tg_set_weights(Engine *e, const float *weights) {
+    return guarded([&] {
+        if (!weights)
+            throw std::runtime_error("Missing weights");
+        e->use_device();
+        const size_t n = size_t(e->layout.count);
+        std::vector<uint16_t> high(n), low(n);
+        for (size_t i = 0; i < n; ++i) {
+            uint32_t bits;
+            std::memcpy(&bits, weights + i, 4);
+            high[i] = uint16_t(bits >> 16);
+            low[i] = uint16_t(bits);
+        }
+        e->upload(e->weight_hi, high.data(), n);
+        e->upload(e->weight_lo, low.data(), n);
+        check_hip(hipMemsetAsync(e->momentum, 0, n * 4, e->stream));
+        check_hip(hipMemsetAsync(e->variance, 0, n * 4, e->stream));
+        e->step = 0;
+        e->sync();
+    });
+}
+// cuda/engine_state.cu:36-55
+TG_API int tg_get_weights(Engine *e, float *weights) {
+    return guarded([&] {
+        if (!weights)
+            throw std::runtime_error("Missing weights output");
+        e->use_device();
+        const size_t n = size_t(e->layout.count);
+        std::vector<uint16_t> high(n), low(n);
+        e->download(high.data(), e->weight_hi, n);
+        e->download(low.data(), e->weight_lo, n);
+        e->sync();
+        for (size_t i = 0; i < n; ++i) {
+            const uint32_t bits = (uint32_t(high[i]) << 16) | low[i];
+            std::memcpy(weights + i, &bits, 4);
+        }
+    });
+}
+TG_API int tg_get_optimizer_state(Engine *e, float *momentum, float *variance, uint64_t *step) {
+    return guarded([&] {
+        if (!momentum || !variance || !step)
+            throw std::runtime_error("Missing optimizer state output");
+        e->use_device();
+        e->download(momentum, e->momentum, size_t(e->layout.count));
+        e->download(variance, e->variance, size_t(e->layout.count));
+        e->sync();
+        *step = e->step;
+    });
+}
+TG_API int tg_set_optimizer_state(Engine *e, const float *momentum, const float *variance, uint64_t step) {
+    return guarded([&] {
+        if (!momentum || !variance)
+            throw std::runtime_error("Missing optimizer state input");
+        e->use_device();
+        e->upload(e->momentum, momentum, size_t(e->layout.count));
+        e->upload(e->variance, variance, size_t(e->layout.count));
+        e->step = step;
+        e->sync();
+    });
+}
+
+TG_API int tg_onecycle_point(const OneCycle *schedule, int step, StepRates *rates) {
+    return guarded([&] {
+        if (!schedule || !rates)
+            throw std::runtime_error("Missing schedule or output");
+        *rates = onecycle_point(*schedule, step);
+    });
+}
+// cuda/runtime.cu:42-61; the table stays on the host because the host issues every optimizer launch
+TG_API int tg_set_onecycle(Engine *e, const OneCycle *schedule) {
+    return guarded([&] {
+        if (!schedule)
+            throw std::runtime_error("Missing schedule");
+        if (!e->schedule.empty() || e->step)
+            throw std::runtime_error("Set OneCycle once, before training");
+        onecycle_point(*schedule, 0); // validate before allocating
+        std::vector<StepRates> rates(size_t(schedule->total_steps));
+        for (int step = 0; step < schedule->total_steps; ++step)
+            rates[size_t(step)] = onecycle_point(*schedule, step);
+        e->schedule = std::move(rates);
+    });
+}
+
+// cuda/runtime.cu:190-206
+TG_API int tg_set_data(Engine *e, const uint8_t *bytes, int64_t size) {
+    return guarded([&] {
+        e->use_device();
+        const int64_t low = std::max(8, e->config.base.context);
+        if (!bytes || size <= low)
+            throw std::runtime_error("Dataset needs at least " + std::to_string(low + 1) + " bytes");
+        if (e->data)
+            throw std::runtime_error("Dataset already loaded");
+        e->allocate(e->data, size_t(size), false);
+        e->data_size = size;
+        e->upload(e->data, bytes, size_t(size));
+        e->sync();
+    });
+}
+
+// cuda/runtime.cu:213-242 with the step loop of cuda/trainer.cuh:109-124 unrolled into launches
+TG_API int tg_train(Engine *e, int steps) {
+    return guarded([&] {
+        if (!e->data || steps < 1 || steps > MaxLaunchSteps)
+            throw std::runtime_error("Load data first; each invocation permits 1.." +
+                                     std::to_string(MaxLaunchSteps) + " steps");
+        if (e->step + uint64_t(steps) > uint64_t(INT_MAX))
+            throw std::runtime_error("Training step count exceeds signed 32-bit indexing");
+        if (!e->schedule.empty() && e->step + uint64_t(steps) > e->schedule.size())
+            throw std::runtime_error("Training would exceed the OneCycle schedule");
+        e->use_device();
+        const Config &c = e->config.base;
+        for (int i = 0; i < steps; ++i) {
+            const uint64_t at = e->step + uint64_t(i);
+            ok(tgk_sample_batch(e->stream, e->data, e->data_size, c.seed, at, c.batch, c.context, e->input,
+                                e->target));
+            e->forward(e->input, e->target, true, nullptr);
+            ok(tgk_position_means(e->stream, e->token_losses, c.batch, c.context,
+                                  e->loss_history + size_t(i) * c.context));
+            e->backward(e->input);
+            e->optimize(at);
+        }
+        e->last_train_steps = steps;
+        e->step += uint64_t(steps);
+    });
+}
+// cuda/engine_state.cu:76-92
+TG_API int tg_get_training_losses(Engine *e, float *losses, int count) {
+    return guarded([&] {
+        if (!losses && count)
+            throw std::runtime_error("Missing training loss output");
+        if (count < 0 || count > e->last_train_steps)
+            throw std::runtime_error("Training loss count exceeds the last launch");
+        e->use_device();
+        e->download(losses, e->loss_history, size_t(count) * e->config.base.context);
+        e->sync();
+    });
+}
+// cuda/runtime.cu:243-262: synchronous engines train step s on weight version s
+TG_API int tg_training_versions(Engine *e, int *out, int count) {
+    return guarded([&] {
+        if (count < 0 || count > e->last_train_steps || (!out && count))
+            throw std::runtime_error("Version trace exceeds last training launch");
+        for (int i = 0; i < count; ++i)
+            out[i] = int(e->step) - e->last_train_steps + i;
+    });
+}
+TG_API int tg_pipeline_stats(Engine *, double *mean, int *maximum) {
+    return guarded([&] {
+        if (!mean || !maximum)
+            throw std::runtime_error("Missing pipeline statistics output");
+        *mean = 0;
+        *maximum = 0;
+    });
+}
+
+// cuda/runtime.cu:291-320
+TG_API int tg_batch(Engine *e, const uint8_t *x, const uint8_t *y, float *logits, float *gradient,
+                    float *loss) {
+    return guarded([&] {
+        if (!x || !y || !logits || !loss)
+            throw std::runtime_error("Missing batch input or output");
+        e->use_device();
+        const size_t M = size_t(e->tokens()), V = size_t(e->config.vocab);
+        if (!e->logits_f32)
+            e->allocate(e->logits_f32, M * V, false);
+        e->upload(e->input, x, M);
+        e->upload(e->target, y, M);
+        e->forward(e->input, e->target, gradient != nullptr, e->logits_f32);
+        if (gradient)
+            e->backward(e->input);
+        e->download(logits, e->logits_f32, M * V);
+        if (gradient)
+            e->download(gradient, e->gradient, size_t(e->layout.count));
+        e->read_losses(loss);
+    });
+}
+// cuda/runtime.cu:322-351
+TG_API int tg_predict(Engine *e, const uint8_t *context, float *logits) {
+    return guarded([&] {
+        if (!context || !logits)
+            throw std::runtime_error("Missing prediction input or output");
+        e->use_device();
+        const Config &c = e->config.base;
+        const size_t M = size_t(e->tokens()), V = size_t(e->config.vocab);
+        if (!e->logits_f32)
+            e->allocate(e->logits_f32, M * V, false);
+        std::vector<uint8_t> input(M), target(M, 0);
+        for (int b = 0; b < c.batch; ++b)
+            std::copy(context, context + c.context, input.begin() + size_t(b) * c.context);
+        e->upload(e->input, input.data(), M);
+        e->upload(e->target, target.data(), M);
+        e->forward(e->input, e->target, false, e->logits_f32);
+        e->download(logits, e->logits_f32 + size_t(c.context - 1) * V, V);
+        e->sync();
+    });
+}
+// cuda/runtime.cu:352-371
+TG_API int tg_optimizer_test(Engine *e, const float *gradient, int steps) {
+    return guarded([&] {
+        if (!gradient)
+            throw std::runtime_error("Missing gradient");
+        if (steps < 1 || steps > 64)
+            throw std::runtime_error("steps must be 1..64");
+        if (!e->schedule.empty() && e->step + uint64_t(steps) > e->schedule.size())
+            throw std::runtime_error("Optimizer test would exceed the OneCycle schedule");
+        e->use_device();
+        e->upload(e->gradient, gradient, size_t(e->layout.count));
+        for (int i = 0; i < steps; ++i)
+            e->optimize(e->step + uint64_t(i));
+        e->step += uint64_t(steps);
+        e->sync();
+    });
+}
