@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Headline benchmark: training tokens/sec of the byte-level GPT d768 L12 H12 T1024 B16
+(BASELINE.json configs[3]) on one MI355X, through the tg_* C ABI.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--kernels]
+
+Prints ONE JSON line.  A step = sample a batch on the GPU, forward, backward, gradient norm, AdamW
+(nothing skipped; inputs are resident in HBM before the timed region).  After the timed region the
+same step is run with a HIP event pair around every operator launch (tg_profile_step) to attribute
+time per operator class; `roofline` describes the dominant MFMA kernel class from those live
+measurements.  `cpu_baseline` times the CPU checker (oracle/, a port - the reference has no CPU
+path) on the host cores for a bounded sample of the same workload.  With --kernels, further JSON
+lines for the isolated GEMM sweep (configs[1]) and attention (configs[2]) go to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+D, L, H, T, B, V = 768, 12, 12, 1024, 16, 256
+F = 4 * D
+M = B * T
+
+
+def gemm_flops():
+    """Algorithmic FLOPs of one launch of each block projection (2*M*N*K), per layer."""
+    shapes = [(3 * D, D), (D, D), (F, D), (D, F)]  # (N, K): qkv, attention-out, mlp-up, mlp-down
+    return [2.0 * M * n * k for n, k in shapes]
+
+
+def class_work():
+    """Algorithmic work per training step for every operator class: ('flop'|'byte', amount)."""
+    per_layer = sum(gemm_flops())
+    attn_fwd = 4.0 * B * H * T * T * 64 / 2  # causal-counted
+    act, wide = M * D * 2, M * F * 2
+    params = V * D * 2 + T * D + L * (4 * D + 4 * D * D + 2 * F * D) + 2 * D
+    return {
+        "gemm_fwd": ("flop", L * per_layer),
+        "gemm_dgrad": ("flop", L * per_layer),
+        "gemm_wgrad": ("flop", L * per_layer),
+        "attn_fwd": ("flop", L * attn_fwd),
+        "attn_bwd": ("flop", L * attn_fwd * 2.5),
+        "head": ("flop", 3 * 2.0 * M * V * D),
+        "layernorm_fwd": ("byte", (2 * L + 1) * 2 * act),
+        "layernorm_bwd": ("byte", (2 * L + 1) * 3 * act + 2 * L * act),  # x, dy, dx (+ residual read)
+        "optimizer": ("byte", params * 28.0 + params * 4.0),            # AdamW 28 B/param + norm pass
+        "other": ("byte", 4 * act + 3 * M * V * 2),
+    }, params
+
+
+def synthetic_weights(layout_count, rng):
+    """N(0, 0.02) matrices, residual-writing ones scaled by 1/sqrt(2L), gamma = 1, beta = 0."""
+    w = np.empty(layout_count, np.float32)
+    n = 0
+
+    def take(size, scale=None, fill=None):
+        nonlocal n
+        if fill is None:
+            w[n:n + size] = rng.standard_normal(size, dtype=np.float32) * scale
+        else:
+            w[n:n + size] = fill
+        n += size
+
+    inner = 0.02 / np.sqrt(2 * L)
+    take(V * D, 0.02)
+    take(T * D, 0.02)
+    for _ in range(L):
+        take(D, fill=1.0), take(D, fill=0.0)
+        take(3 * D * D, 0.02), take(D * D, inner)
+        take(D, fill=1.0), take(D, fill=0.0)
+        take(F * D, 0.02), take(D * F, inner)
+    take(D, fill=1.0), take(D, fill=0.0)
+    take(V * D, 0.02)
+    assert n == layout_count
+    return w
+
+
+def zipf_bytes(n, rng, s=1.1):
+    p = np.arange(1, 257, dtype=np.float64) ** -s
+    cdf = np.cumsum(p / p.sum())
+    return np.minimum(np.searchsorted(cdf, rng.random(n)), 255).astype(np.uint8)
+
+
+def cpu_baseline():
+    """The CPU checker on one of the step's 16 sequences (same model, B=1): forward, backward, AdamW."""
+    import oracle
+    cfg = oracle.model(depth=L, context=T, batch=1, d_model=D, heads=H)
+    w = oracle.init_weights(cfg)
+    z = np.zeros_like(w)
+    data = oracle.fill_zipf_bytes(1 << 16, 71)
+    start = time.perf_counter()
+    oracle.train(cfg, w, z, z, data, 3407, 0, 1, 3e-4, 0.9, 0.95, 1e-8, 0.1, 1.0)
+    seconds = time.perf_counter() - start
+    return {"value": T / seconds, "unit": "tokens/s", "cores": oracle.threads(), "kind": "port",
+            "sample": f"one training step of the same model on 1 of the {B} sequences (B=1, T={T}): "
+                      f"{seconds:.1f} s of the fp32 OpenMP checker (oracle/tg_oracle.c)"}
+
+
+def kernel_sweeps(out):
+    """configs[1] (GEMM sweep, M=16384) and configs[2] (attention B16 H12 T1024) through tgk_*."""
+    import torch
+    from turbogpt_amd.bridge import check, library
+    lib = library()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def timed(fn, iters=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters
+
+    for k, n in [(768, 2304), (768, 768), (768, 3072), (3072, 768)]:
+        x = torch.randn(M, k, device="cuda").bfloat16()
+        w = torch.randn(n, k, device="cuda").bfloat16()
+        dy = torch.randn(M, n, device="cuda").bfloat16()
+        y = torch.empty(M, n, device="cuda", dtype=torch.bfloat16)
+        dx = torch.empty(M, k, device="cuda", dtype=torch.bfloat16)
+        dw = torch.empty(n, k, device="cuda")
+        need = lib.tgk_gemm_wgrad_workspace(M, n, k)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        flop = 2.0 * M * n * k
+        runs = {
+            "fwd": lambda: check(lib.tgk_gemm_fwd(stream, M, n, k, x.data_ptr(), k, w.data_ptr(), k, y.data_ptr(), n,
+                                                  None, 0, None, 0)),
+            "dgrad": lambda: check(lib.tgk_gemm_dgrad(stream, M, n, k, dy.data_ptr(), n, w.data_ptr(), k,
+                                                      dx.data_ptr(), k, None, 0)),
+            "wgrad": lambda: check(lib.tgk_gemm_wgrad(stream, M, n, k, dy.data_ptr(), n, x.data_ptr(), k,
+                                                      dw.data_ptr(), k, 0, ws.data_ptr(), need)),
+        }
+        for name, fn in runs.items():
+            ms = timed(fn)
+            print(json.dumps({"kernel": f"gemm_{name}", "M": M, "K": k, "N": n, "ms": round(ms, 4),
+                              "tflops": round(flop / ms / 1e9, 1),
+                              "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
+    d = H * 64
+    qkv = torch.randn(M, 3 * d, device="cuda").bfloat16()
+    do = torch.randn(M, d, device="cuda").bfloat16()
+    o = torch.empty(M, d, device="cuda", dtype=torch.bfloat16)
+    lse = torch.empty(B, H, T, device="cuda")
+    dqkv = torch.empty_like(qkv)
+    need = lib.tgk_attn_bwd_workspace(B, H, T)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    p, g = qkv.data_ptr(), dqkv.data_ptr()
+    flop = 4.0 * B * H * T * T * 64 / 2
+    ms = timed(lambda: check(lib.tgk_attn_fwd(stream, B, H, T, 64, p, p + 2 * d, p + 4 * d, 3 * d, o.data_ptr(), d,
+                                              lse.data_ptr(), 0.125)))
+    print(json.dumps({"kernel": "attn_fwd", "B": B, "H": H, "T": T, "ms": round(ms, 4),
+                      "tflops_causal_counted": round(flop / ms / 1e9, 1),
+                      "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
+    ms = timed(lambda: check(lib.tgk_attn_bwd(stream, B, H, T, 64, p, p + 2 * d, p + 4 * d, 3 * d, o.data_ptr(), d,
+                                              lse.data_ptr(), do.data_ptr(), d, g, g + 2 * d, g + 4 * d, 3 * d, 0.125,
+                                              ws.data_ptr(), need)))
+    print(json.dumps({"kernel": "attn_bwd", "B": B, "H": H, "T": T, "ms": round(ms, 4),
+                      "tflops_causal_counted": round(2.5 * flop / ms / 1e9, 1),
+                      "frac_of_bf16_peak": round(2.5 * flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernels", action="store_true", help="also print the isolated kernel sweeps to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures one GPU (the engine is single-device); run with --gpus 1")
+    if not 1 <= args.steps <= 4096 or not 0 <= args.warmup <= 4096:
+        sys.exit("bench.py: steps must be 1..4096 and warmup 0..4096 (one tg_train call each)")
+
+    if args.kernels:
+        # torch ships its own HIP runtime: it has to be the first one loaded in this process
+        import torch
+        torch.cuda.init()
+    from turbogpt_amd.bridge import ModelConfig, Native
+    cfg = ModelConfig(d_model=D, depth=L, context=T, batch=B, heads=H, ffn=F, learning_rate=3e-4, beta1=0.9,
+                      beta2=0.95, weight_decay=0.1, clip=1.0, seed=3407)
+    rng = np.random.default_rng(3407)
+    with Native(cfg) as engine:
+        engine.set_weights(synthetic_weights(engine.count, rng))
+        engine.set_data(zipf_bytes(1 << 24, np.random.default_rng(71)))
+        if args.warmup:
+            engine.train(args.warmup)
+        engine.synchronize()
+        start = time.perf_counter()
+        engine.train(args.steps)
+        engine.synchronize()
+        seconds = time.perf_counter() - start
+        losses = engine.training_losses(args.steps).mean(1)
+
+        work, params = class_work()
+        profile = {}
+        for _ in range(3):
+            for name, (ms, launches) in engine.profile_step().items():
+                total, count = profile.get(name, (0.0, 0))
+                profile[name] = (total + ms, count + launches)
+    classes = {}
+    for name, (ms, launches) in profile.items():
+        kind, amount = work[name]
+        per_step_ms = ms / 3
+        rate = amount / (per_step_ms * 1e-3) / 1e12 if per_step_ms > 0 else 0.0
+        classes[name] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // 3,
+                         ("tflops" if kind == "flop" else "tb_per_s"): round(rate, 2)}
+    # dominant MFMA kernel: the forward block-projection GEMM (one template instantiation, 4 launches/layer)
+    fwd_ms, fwd_launches = profile["gemm_fwd"]
+    flops_per_launch = sum(gemm_flops()) / 4
+    achieved = flops_per_launch / (fwd_ms / fwd_launches * 1e-3) / 1e12
+    ms_per_step = seconds / args.steps * 1e3
+    result = {
+        "metric": "train tokens/sec at d768 L12 T1024 (1 GPU)",
+        "value": round(args.steps * M / seconds, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[3]: full training step, byte-level GPT d_model=768 L=12 H=12 T=1024 B=16 "
+                               "ffn=3072 vocab=256, bf16 weights with fp32 masters, AdamW lr 3e-4 betas 0.9/0.95 "
+                               "wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
+                   "global_batch": B, "seq_len": T, "parameters": params, "parallelism": "single GPU"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<256,192,kcontig,kcontig,EpilogueBf16> (forward "
+                     "block projections)", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "flops_per_launch": flops_per_launch,
+                     "avg_launch_ms": round(fwd_ms / fwd_launches, 5)},
+        "classes": classes,
+        # 9.45 TFLOP of algorithmic work per step (attention causal-counted, backward = 2.5 x forward)
+        "model_tflops": round((3 * L * sum(gemm_flops()) + 3 * 2.0 * M * V * D +
+                               L * 3.5 * 4.0 * B * H * T * T * 64 / 2) / (ms_per_step * 1e-3) / 1e12, 1),
+        "loss_first_last": [round(float(losses[0]), 4), round(float(losses[-1]), 4)],
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    if args.kernels:
+        kernel_sweeps(sys.stderr)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -87,6 +87,24 @@ TG_API int tg_predict(Engine *engine, const uint8_t *context, float *logits); /*
 TG_API int tg_optimizer_test(Engine *engine, const float *gradients, int steps); /* 1..64 */
 TG_API int tg_synchronize(Engine *engine);
 
+/* Not in the reference: measurement aid.  Runs one training step exactly like tg_train(engine, 1)
+ * with a HIP event pair around every operator launch on the engine's stream, and returns summed
+ * milliseconds and launch counts per operator class.  Synchronises. */
+enum {
+    TG_CLASS_GEMM_FWD = 0,   /* block projections forward (QKV, attention-out, MLP-up, MLP-down) */
+    TG_CLASS_GEMM_DGRAD = 1, /* their input gradients */
+    TG_CLASS_GEMM_WGRAD = 2, /* their weight gradients, split-K reduction included */
+    TG_CLASS_ATTN_FWD = 3,
+    TG_CLASS_ATTN_BWD = 4,
+    TG_CLASS_LAYERNORM_FWD = 5,
+    TG_CLASS_LAYERNORM_BWD = 6,
+    TG_CLASS_HEAD = 7,       /* vocabulary projection: forward, dgrad, wgrad */
+    TG_CLASS_OTHER = 8,      /* sampling, embedding, cross-entropy, loss means */
+    TG_CLASS_OPTIMIZER = 9,  /* gradient norm + AdamW */
+    TG_CLASSES = 10
+};
+TG_API int tg_profile_step(Engine *engine, float *class_ms, int *class_launches, int classes);
+
 #ifdef __cplusplus
 static_assert(sizeof(Config) == 72, "Config must keep the reference layout");
 static_assert(sizeof(OneCycle) == 48 && sizeof(StepRates) == 8, "schedule PODs must keep the reference layout");

@@ -84,9 +84,12 @@ TGK_API size_t tgk_attn_bwd_workspace(int B, int H, int T);
 TGK_API int tgk_embed_fwd(hipStream_t stream, int rows, int T, int D, const uint8_t *x,
                           const uint16_t *table, const uint16_t *positions, uint16_t *out);
 /* dtable[v] (=|+=) sum_{t: x[t]=v} dh[t]; dpositions[p] (=|+=) sum_b dh[b*T+p]; fp32.  Replaces
- * the atomicAdd scatter of cuda/model.cuh:96-97 with a fixed-order sum. D multiple of 64. */
+ * the atomicAdd scatter of cuda/model.cuh:96-97 with a fixed-order sum. D multiple of 64, vocab
+ * 256.  workspace: tgk_embed_bwd_workspace(B*T, D) bytes. */
 TGK_API int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab, const uint8_t *x,
-                          const uint16_t *dh, float *dtable, float *dpositions, int accumulate);
+                          const uint16_t *dh, float *dtable, float *dpositions, int accumulate,
+                          void *workspace, size_t workspace_bytes);
+TGK_API size_t tgk_embed_bwd_workspace(int rows, int D);
 
 /* y = RN_bf16((x - mean) * rsqrt(var + eps) * gamma + beta) per row; takes the slot of normalize
  * (cuda/ops.cuh:57-66; RMSNorm there, LayerNorm in the target model). D multiple of 8, <= 2048. */
@@ -95,7 +98,7 @@ TGK_API int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint16_
                               const uint16_t *beta_hi, const uint16_t *beta_lo, uint16_t *y, float eps);
 /* dx = RN_bf16(LN'(x) dy), or with residual != 0: dx = RN_bf16(dx + RN_bf16(LN'(x) dy)) (residual
  * gradients stay in bf16, cuda/ops.cuh:74-76); dgamma/dbeta (=|+=) fixed-order column sums in
- * fp32 (replaces the atomicAdd of cuda/ops.cuh:77).  Takes the slot of norm_backward
+ * fp32 (replaces the atomicAdd of cuda/ops.cuh:77); D multiple of 64.  Takes the slot of norm_backward
  * (cuda/ops.cuh:67-80).  workspace: tgk_layernorm_bwd_workspace(rows, D) bytes. */
 TGK_API int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint16_t *x, const uint16_t *dy,
                               const uint16_t *gamma_hi, const uint16_t *gamma_lo, uint16_t *dx,

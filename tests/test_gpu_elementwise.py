@@ -22,7 +22,7 @@ def hilo(orc, w):
     return dev(hi.view(np.int16)), dev(lo.view(np.int16))
 
 
-@pytest.mark.parametrize("B,T,D", [(2, 128, 256), (3, 64, 768)])
+@pytest.mark.parametrize("B,T,D", [(2, 128, 256), (3, 64, 768), (9, 256, 128)])
 def test_embedding_forward_and_backward(orc, B, T, D):
     lib = library()
     rng = np.random.default_rng(B + T + D)
@@ -38,13 +38,17 @@ def test_embedding_forward_and_backward(orc, B, T, D):
     dh, dhh = to_bf16_device(rng.standard_normal((B * T, D)))
     dt = torch.full((256, D), 1.0, dtype=torch.float32, device="cuda")
     dp = torch.full((T, D), 1.0, dtype=torch.float32, device="cuda")
-    check(lib.tgk_embed_bwd(stream(), B, T, D, 256, xd.data_ptr(), dh.data_ptr(), dt.data_ptr(), dp.data_ptr(), 0))
+    need = lib.tgk_embed_bwd_workspace(B * T, D)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    check(lib.tgk_embed_bwd(stream(), B, T, D, 256, xd.data_ptr(), dh.data_ptr(), dt.data_ptr(), dp.data_ptr(), 0,
+                            ws.data_ptr(), need))
     sync()
     want_t = np.zeros((256, D), np.float64)
     np.add.at(want_t, x, dhh.astype(np.float64))
     assert rel(host(dt), want_t) < 1e-6
     assert rel(host(dp), dhh.reshape(B, T, D).astype(np.float64).sum(0)) < 1e-6
-    check(lib.tgk_embed_bwd(stream(), B, T, D, 256, xd.data_ptr(), dh.data_ptr(), dt.data_ptr(), dp.data_ptr(), 1))
+    check(lib.tgk_embed_bwd(stream(), B, T, D, 256, xd.data_ptr(), dh.data_ptr(), dt.data_ptr(), dp.data_ptr(), 1,
+                            ws.data_ptr(), need))
     sync()
     assert rel(host(dt), 2 * want_t) < 1e-6
 

@@ -25,7 +25,8 @@ KERNEL_ABI = {
                            f32, vp, sz]),
     "tgk_attn_bwd_workspace": (sz, [i32, i32, i32]),
     "tgk_embed_fwd": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
-    "tgk_embed_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32]),
+    "tgk_embed_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32, vp, sz]),
+    "tgk_embed_bwd_workspace": (sz, [i32, i32]),
     "tgk_layernorm_fwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, f32]),
     "tgk_layernorm_bwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, f32, i32, i32, vp, sz]),
     "tgk_layernorm_bwd_workspace": (sz, [i32, i32]),
@@ -102,7 +103,10 @@ ENGINE_ABI = {
     "tg_predict": (i32, [vp, vp, vp]),
     "tg_optimizer_test": (i32, [vp, vp, i32]),
     "tg_synchronize": (i32, [vp]),
+    "tg_profile_step": (i32, [vp, vp, vp, i32]),
 }
+CLASSES = ("gemm_fwd", "gemm_dgrad", "gemm_wgrad", "attn_fwd", "attn_bwd", "layernorm_fwd", "layernorm_bwd",
+           "head", "other", "optimizer")
 
 
 def library_path():
@@ -199,6 +203,13 @@ class Native:
         grad = self.np.ascontiguousarray(grad, dtype=self.np.float32)
         assert grad.size == self.count
         self.check(self.lib.tg_optimizer_test(self.handle, grad.ctypes.data, steps))
+
+    def profile_step(self):
+        """One training step with per-class HIP-event timing: {class: (milliseconds, launches)}."""
+        ms = (C.c_float * len(CLASSES))()
+        launches = (C.c_int * len(CLASSES))()
+        self.check(self.lib.tg_profile_step(self.handle, ms, launches, len(CLASSES)))
+        return {name: (ms[i], launches[i]) for i, name in enumerate(CLASSES)}
 
     def synchronize(self):
         self.check(self.lib.tg_synchronize(self.handle))

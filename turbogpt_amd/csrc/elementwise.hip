@@ -59,34 +59,38 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(const uint8_t *__restric
     }
 }
 
-// dTable[v][c] = sum over tokens t with x[t] == v of dh[t][c], in token order.
-// grid (vocab, D/64); 256 threads = 4 token phases x 64 columns.
-__global__ __launch_bounds__(256) void embed_bwd_table_kernel(const uint8_t *__restrict__ x,
-                                                              const bf16_t *__restrict__ dh,
-                                                              float *__restrict__ dtable, int rows,
-                                                              int D, int accumulate) {
-    __shared__ uint8_t tokens[4096];
-    __shared__ float part[4][64];
-    const int v = blockIdx.x, col = blockIdx.y * 64 + (threadIdx.x & 63), phase = threadIdx.x >> 6;
-    float sum = 0.f;
-    for (int base = 0; base < rows; base += 4096) {
-        const int n = rows - base < 4096 ? rows - base : 4096;
-        __syncthreads();
-        for (int i = threadIdx.x; i < n; i += 256)
-            tokens[i] = x[base + i];
-        __syncthreads();
-        for (int i = phase; i < n; i += 4)
-            if (tokens[i] == v)
-                sum += bf16_to_float(dh[size_t(base + i) * D + col]);
-    }
-    part[phase][threadIdx.x & 63] = sum;
+// dTable[v][c] = sum over tokens t with x[t] == v of dh[t][c].  Pass 1: one wave per (64 columns,
+// token segment) walks its segment in token order and adds each row slice into a [256][64] fp32
+// table in LDS (each lane owns one column, LDS adds retire in program order: fixed summation
+// order), then dumps the table.  Pass 2 folds the segment tables in segment order.
+constexpr int EMBED_SEGMENT = 1024; // tokens per segment
+__global__ __launch_bounds__(64) void embed_bwd_partial_kernel(const uint8_t *__restrict__ x,
+                                                               const bf16_t *__restrict__ dh,
+                                                               float *__restrict__ partial, int rows, int D) {
+    __shared__ float table[256 * 64];
+    const int lane = threadIdx.x, col = blockIdx.x * 64 + lane, segment = blockIdx.y;
+    for (int i = lane; i < 256 * 64; i += 64)
+        table[i] = 0.f;
     __syncthreads();
-    if (phase == 0) {
-        const int c = threadIdx.x;
-        float total = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
-        float *p = dtable + size_t(v) * D + col;
-        *p = accumulate ? *p + total : total;
-    }
+    const int begin = segment * EMBED_SEGMENT, end = begin + EMBED_SEGMENT < rows ? begin + EMBED_SEGMENT : rows;
+#pragma unroll 8
+    for (int t = begin; t < end; ++t)
+        atomicAdd(&table[int(x[t]) * 64 + lane], bf16_to_float(dh[size_t(t) * D + col]));
+    __syncthreads();
+    float *out = partial + size_t(segment) * 256 * D + col;
+    for (int v = 0; v < 256; ++v)
+        out[size_t(v) * D] = table[v * 64 + lane];
+}
+__global__ __launch_bounds__(256) void embed_bwd_fold_kernel(const float *__restrict__ partial, int segments,
+                                                             float *__restrict__ dtable, size_t count,
+                                                             int accumulate) {
+    const size_t i = blockIdx.x * size_t(256) + threadIdx.x;
+    if (i >= count)
+        return;
+    float sum = 0.f;
+    for (int s = 0; s < segments; ++s)
+        sum += partial[size_t(s) * count + i];
+    dtable[i] = accumulate ? dtable[i] + sum : sum;
 }
 // dPositions[p][c] = sum over sequences b of dh[b*T + p][c]
 __global__ __launch_bounds__(256) void embed_bwd_positions_kernel(const bf16_t *__restrict__ dh,
@@ -250,20 +254,32 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
         partial[size_t(blockIdx.x) * 2 * D + i] =
             (lds[i] + lds[2 * D + i]) + (lds[4 * D + i] + lds[6 * D + i]);
 }
-// dgamma[c] (+)= sum_b partial[b][0][c], dbeta likewise; fixed order over b
+// dgamma[c] (+)= sum_b partial[b][0][c], dbeta likewise.  64 columns per block, 4 interleaved
+// block phases per column combined in a fixed order.
 __global__ __launch_bounds__(256) void layernorm_bwd_reduce_kernel(const float *__restrict__ partial,
                                                                    int blocks, int D,
                                                                    float *__restrict__ dgamma,
                                                                    float *__restrict__ dbeta,
                                                                    int accumulate) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= 2 * D)
-        return;
-    float sum = 0.f;
-    for (int b = 0; b < blocks; ++b)
-        sum += partial[size_t(b) * 2 * D + i];
-    float *out = i < D ? dgamma + i : dbeta + (i - D);
-    *out = accumulate ? *out + sum : sum;
+    __shared__ float part[4][64];
+    const int col = threadIdx.x & 63, phase = threadIdx.x >> 6, i = blockIdx.x * 64 + col;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int b = phase;
+    for (; b + 12 < blocks; b += 16) { // four independent loads in flight per thread
+        s0 += partial[size_t(b) * 2 * D + i];
+        s1 += partial[size_t(b + 4) * 2 * D + i];
+        s2 += partial[size_t(b + 8) * 2 * D + i];
+        s3 += partial[size_t(b + 12) * 2 * D + i];
+    }
+    for (; b < blocks; b += 4)
+        s0 += partial[size_t(b) * 2 * D + i];
+    part[phase][col] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (phase == 0) {
+        const float sum = (part[0][col] + part[1][col]) + (part[2][col] + part[3][col]);
+        float *out = i < D ? dgamma + i : dbeta + (i - D);
+        *out = accumulate ? *out + sum : sum;
+    }
 }
 
 // ---- cross-entropy over 256 byte classes ------------------------------------------------------
@@ -452,14 +468,27 @@ extern "C" int tgk_embed_fwd(hipStream_t stream, int rows, int T, int D, const u
     });
 }
 
+extern "C" size_t tgk_embed_bwd_workspace(int rows, int D) {
+    if (rows <= 0 || D <= 0)
+        return 0;
+    return size_t((rows + EMBED_SEGMENT - 1) / EMBED_SEGMENT) * 256 * D * sizeof(float);
+}
 extern "C" int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab, const uint8_t *x,
-                             const uint16_t *dh, float *dtable, float *dpositions, int accumulate) {
+                             const uint16_t *dh, float *dtable, float *dpositions, int accumulate,
+                             void *workspace, size_t workspace_bytes) {
     return guarded([&] {
         require(B > 0 && T > 0 && D > 0 && D % 64 == 0, "embed_bwd: D must be a positive multiple of 64");
-        require(vocab > 0 && vocab <= 256, "embed_bwd: vocabulary is at most 256 (byte tokens)");
+        require(vocab == 256, "embed_bwd: vocabulary must be 256 (byte tokens)");
         require(x && dh && dtable && dpositions, "embed_bwd: missing operand");
-        hipLaunchKernelGGL(embed_bwd_table_kernel, dim3(vocab, D / 64), dim3(256), 0, stream, x, dh, dtable,
-                           B * T, D, accumulate);
+        const int rows = B * T, segments = (rows + EMBED_SEGMENT - 1) / EMBED_SEGMENT;
+        require(workspace && workspace_bytes >= tgk_embed_bwd_workspace(rows, D),
+                "embed_bwd: workspace too small (see tgk_embed_bwd_workspace)");
+        float *partial = static_cast<float *>(workspace);
+        hipLaunchKernelGGL(embed_bwd_partial_kernel, dim3(D / 64, segments), dim3(64), 0, stream, x, dh, partial,
+                           rows, D);
+        const size_t count = size_t(256) * D;
+        hipLaunchKernelGGL(embed_bwd_fold_kernel, dim3(unsigned((count + 255) / 256)), dim3(256), 0, stream, partial,
+                           segments, dtable, count, accumulate);
         hipLaunchKernelGGL(embed_bwd_positions_kernel, dim3(grid_for(size_t(T) * D, 256)), dim3(256), 0, stream,
                            dh, dpositions, B, T, D, accumulate);
         check_hip(hipGetLastError(), "embed_bwd launch: ");
@@ -485,7 +514,7 @@ extern "C" int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint
 }
 
 static int layernorm_bwd_blocks(int rows) {
-    return grid_for(rows, 16, 1024);
+    return grid_for(rows, 16, 512);
 }
 extern "C" size_t tgk_layernorm_bwd_workspace(int rows, int D) {
     return rows > 0 && D > 0 ? size_t(layernorm_bwd_blocks(rows)) * 2 * D * sizeof(float) : 0;
@@ -495,8 +524,8 @@ extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint
                                  uint16_t *dx, float *dgamma, float *dbeta, float eps, int residual,
                                  int accumulate, void *workspace, size_t workspace_bytes) {
     return guarded([&] {
-        require(rows > 0 && D > 0 && D % 8 == 0 && D <= MAX_LN_CHUNKS * 512,
-                "layernorm: D must be a multiple of 8, at most 2048");
+        require(rows > 0 && D > 0 && D % 64 == 0 && D <= MAX_LN_CHUNKS * 512,
+                "layernorm_bwd: D must be a multiple of 64, at most 2048");
         aligned(x, "layernorm: x");
         aligned(dy, "layernorm: dy");
         aligned(dx, "layernorm: dx");
@@ -509,8 +538,8 @@ extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint
         float *partial = static_cast<float *>(workspace);
         hipLaunchKernelGGL(layernorm_bwd_kernel, dim3(blocks), dim3(256), size_t(8) * D * sizeof(float), stream, x,
                            dy, gamma_hi, gamma_lo, dx, partial, rows, D, eps, residual);
-        hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3((2 * D + 255) / 256), dim3(256), 0, stream, partial,
-                           blocks, D, dgamma, dbeta, accumulate);
+        hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3(2 * D / 64), dim3(256), 0, stream, partial, blocks, D,
+                           dgamma, dbeta, accumulate);
         check_hip(hipGetLastError(), "layernorm_bwd launch: ");
     });
 }

@@ -26,6 +26,12 @@ void ok(int status) {
     if (status < 0)
         throw std::runtime_error(tg_last_error);
 }
+// one operator launch, attributed to a TG_CLASS_* for tg_profile_step
+#define OP(cls, call)                 \
+    do {                              \
+        Scope profile_scope(this, cls); \
+        ok(call);                     \
+    } while (0)
 
 // optim.h:18-44
 StepRates onecycle_point(const OneCycle &s, int step) {
@@ -79,6 +85,40 @@ struct Engine {
     uint64_t step = 0;
     int last_train_steps = 0;
 
+    // optional per-class timing of one step (tg_profile_step): event pairs around every launch
+    struct Span {
+        int cls;
+        hipEvent_t start, stop;
+    };
+    bool profiling = false;
+    std::vector<Span> spans;
+    std::vector<hipEvent_t> event_pool;
+    hipEvent_t event() {
+        if (event_pool.empty()) {
+            hipEvent_t fresh;
+            check_hip(hipEventCreate(&fresh));
+            return fresh;
+        }
+        hipEvent_t pooled = event_pool.back();
+        event_pool.pop_back();
+        return pooled;
+    }
+    struct Scope {
+        Engine *e;
+        size_t index = 0;
+        Scope(Engine *engine, int cls) : e(engine) {
+            if (!e->profiling)
+                return;
+            index = e->spans.size();
+            e->spans.push_back({cls, e->event(), e->event()});
+            check_hip(hipEventRecord(e->spans[index].start, e->stream));
+        }
+        ~Scope() {
+            if (e->profiling)
+                (void)hipEventRecord(e->spans[index].stop, e->stream);
+        }
+    };
+
     int tokens() const { return config.base.batch * config.base.context; }
 
     template <class T> void allocate(T *&ptr, size_t n, bool zero = true) { // cuda/engine_internal.h:17-27
@@ -104,6 +144,12 @@ struct Engine {
             (void)hipStreamSynchronize(stream);
         for (void *allocation : allocations)
             (void)hipFree(allocation);
+        for (Span &span : spans) {
+            (void)hipEventDestroy(span.start);
+            (void)hipEventDestroy(span.stop);
+        }
+        for (hipEvent_t pooled : event_pool)
+            (void)hipEventDestroy(pooled);
         if (stream)
             (void)hipStreamDestroy(stream);
     }
@@ -116,25 +162,25 @@ struct Engine {
         const Config &c = config.base;
         const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
-        ok(tgk_embed_fwd(stream, M, T, d, tokens_in, w(layout.embedding), w(layout.positions), x[0]));
+        OP(TG_CLASS_OTHER, tgk_embed_fwd(stream, M, T, d, tokens_in, w(layout.embedding), w(layout.positions), x[0]));
         for (int l = 0; l < c.depth; ++l) {
             const TgLayerParameters &p = layout.layers[l];
             LayerBuffers &b = layers[l];
-            ok(tgk_layernorm_fwd(stream, M, d, x[l], w(p.ln1_g), wl(p.ln1_g), w(p.ln1_b), wl(p.ln1_b), b.n1,
+            OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, x[l], w(p.ln1_g), wl(p.ln1_g), w(p.ln1_b), wl(p.ln1_b), b.n1,
                                  config.ln_eps));
-            ok(tgk_gemm_fwd(stream, M, 3 * d, d, b.n1, d, w(p.qkv), d, b.qkv, 3 * d, nullptr, 0, nullptr, 0));
-            ok(tgk_attn_fwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, 3 * d, d, b.n1, d, w(p.qkv), d, b.qkv, 3 * d, nullptr, 0, nullptr, 0));
+            OP(TG_CLASS_ATTN_FWD, tgk_attn_fwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
                             3 * d, b.o, d, b.lse, scale));
-            ok(tgk_gemm_fwd(stream, M, d, d, b.o, d, w(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
-            ok(tgk_layernorm_fwd(stream, M, d, b.mid, w(p.ln2_g), wl(p.ln2_g), w(p.ln2_b), wl(p.ln2_b), b.n2,
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, d, b.o, d, w(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
+            OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, b.mid, w(p.ln2_g), wl(p.ln2_g), w(p.ln2_b), wl(p.ln2_b), b.n2,
                                  config.ln_eps));
-            ok(tgk_gemm_fwd(stream, M, F, d, b.n2, d, w(p.mlp_up), d, b.u, F, nullptr, 0, b.a, F));
-            ok(tgk_gemm_fwd(stream, M, d, F, b.a, F, w(p.mlp_down), F, x[l + 1], d, b.mid, d, nullptr, 0));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, F, d, b.n2, d, w(p.mlp_up), d, b.u, F, nullptr, 0, b.a, F));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, F, b.a, F, w(p.mlp_down), F, x[l + 1], d, b.mid, d, nullptr, 0));
         }
-        ok(tgk_layernorm_fwd(stream, M, d, x[c.depth], w(layout.lnf_g), wl(layout.lnf_g), w(layout.lnf_b),
+        OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, x[c.depth], w(layout.lnf_g), wl(layout.lnf_g), w(layout.lnf_b),
                              wl(layout.lnf_b), nf, config.ln_eps));
-        ok(tgk_gemm_fwd(stream, M, V, d, nf, d, w(layout.head), d, logits, V, nullptr, 0, nullptr, 0));
-        ok(tgk_cross_entropy(stream, M, V, logits, targets, token_losses, logits_out, 1.0f / float(M),
+        OP(TG_CLASS_HEAD, tgk_gemm_fwd(stream, M, V, d, nf, d, w(layout.head), d, logits, V, nullptr, 0, nullptr, 0));
+        OP(TG_CLASS_OTHER, tgk_cross_entropy(stream, M, V, logits, targets, token_losses, logits_out, 1.0f / float(M),
                              with_gradient ? 1 : 0));
     }
 
@@ -144,31 +190,32 @@ struct Engine {
         const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
         float *g = gradient;
-        ok(tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
-        ok(tgk_gemm_dgrad(stream, M, V, d, logits, V, w(layout.head), d, t1, d, nullptr, 0));
-        ok(tgk_layernorm_bwd(stream, M, d, x[c.depth], t1, w(layout.lnf_g), wl(layout.lnf_g), dh,
+        OP(TG_CLASS_HEAD, tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
+        OP(TG_CLASS_HEAD, tgk_gemm_dgrad(stream, M, V, d, logits, V, w(layout.head), d, t1, d, nullptr, 0));
+        OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, x[c.depth], t1, w(layout.lnf_g), wl(layout.lnf_g), dh,
                              g + layout.lnf_g, g + layout.lnf_b, config.ln_eps, 0, 0, workspace, workspace_bytes));
         for (int l = c.depth - 1; l >= 0; --l) {
             const TgLayerParameters &p = layout.layers[l];
             LayerBuffers &b = layers[l];
-            ok(tgk_gemm_wgrad(stream, M, d, F, dh, d, b.a, F, g + p.mlp_down, F, 0, workspace, workspace_bytes));
-            ok(tgk_gemm_dgrad(stream, M, d, F, dh, d, w(p.mlp_down), F, du, F, b.u, F));
-            ok(tgk_gemm_wgrad(stream, M, F, d, du, F, b.n2, d, g + p.mlp_up, d, 0, workspace, workspace_bytes));
-            ok(tgk_gemm_dgrad(stream, M, F, d, du, F, w(p.mlp_up), d, t1, d, nullptr, 0));
-            ok(tgk_layernorm_bwd(stream, M, d, b.mid, t1, w(p.ln2_g), wl(p.ln2_g), dh, g + p.ln2_g, g + p.ln2_b,
+            OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, F, dh, d, b.a, F, g + p.mlp_down, F, 0, workspace, workspace_bytes));
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, d, F, dh, d, w(p.mlp_down), F, du, F, b.u, F));
+            OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, F, d, du, F, b.n2, d, g + p.mlp_up, d, 0, workspace, workspace_bytes));
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, F, d, du, F, w(p.mlp_up), d, t1, d, nullptr, 0));
+            OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, b.mid, t1, w(p.ln2_g), wl(p.ln2_g), dh, g + p.ln2_g, g + p.ln2_b,
                                  config.ln_eps, 1, 0, workspace, workspace_bytes));
-            ok(tgk_gemm_wgrad(stream, M, d, d, dh, d, b.o, d, g + p.attn_out, d, 0, workspace, workspace_bytes));
-            ok(tgk_gemm_dgrad(stream, M, d, d, dh, d, w(p.attn_out), d, t1, d, nullptr, 0));
-            ok(tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
+            OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, d, dh, d, b.o, d, g + p.attn_out, d, 0, workspace, workspace_bytes));
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, d, d, dh, d, w(p.attn_out), d, t1, d, nullptr, 0));
+            OP(TG_CLASS_ATTN_BWD, tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
                             3 * d, b.o, d, b.lse, t1, d, dqkv, dqkv + d, dqkv + 2 * d, 3 * d, scale, workspace,
                             workspace_bytes));
-            ok(tgk_gemm_wgrad(stream, M, 3 * d, d, dqkv, 3 * d, b.n1, d, g + p.qkv, d, 0, workspace,
+            OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, 3 * d, d, dqkv, 3 * d, b.n1, d, g + p.qkv, d, 0, workspace,
                               workspace_bytes));
-            ok(tgk_gemm_dgrad(stream, M, 3 * d, d, dqkv, 3 * d, w(p.qkv), d, t1, d, nullptr, 0));
-            ok(tgk_layernorm_bwd(stream, M, d, x[l], t1, w(p.ln1_g), wl(p.ln1_g), dh, g + p.ln1_g, g + p.ln1_b,
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, 3 * d, d, dqkv, 3 * d, w(p.qkv), d, t1, d, nullptr, 0));
+            OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, x[l], t1, w(p.ln1_g), wl(p.ln1_g), dh, g + p.ln1_g, g + p.ln1_b,
                                  config.ln_eps, 1, 0, workspace, workspace_bytes));
         }
-        ok(tgk_embed_bwd(stream, c.batch, T, d, V, tokens_in, dh, g + layout.embedding, g + layout.positions, 0));
+        OP(TG_CLASS_OTHER, tgk_embed_bwd(stream, c.batch, T, d, V, tokens_in, dh, g + layout.embedding, g + layout.positions, 0,
+                                         workspace, workspace_bytes));
     }
 
     // cuda/optim.cuh:66-106 for optimizer step `at` (0-based)
@@ -180,10 +227,19 @@ struct Engine {
             beta1 = schedule[at].momentum;
         }
         if (c.clip > 0)
-            ok(tgk_sumsq_partials(stream, gradient, size_t(layout.count), norm_partials, NormPartials));
-        ok(tgk_adamw(stream, size_t(layout.count), weight_hi, weight_lo, momentum, variance, gradient,
+            OP(TG_CLASS_OPTIMIZER, tgk_sumsq_partials(stream, gradient, size_t(layout.count), norm_partials, NormPartials));
+        OP(TG_CLASS_OPTIMIZER, tgk_adamw(stream, size_t(layout.count), weight_hi, weight_lo, momentum, variance, gradient,
                      norm_partials, NormPartials, segment_starts, segment_flags, segments, lr, beta1, c.beta2,
                      c.epsilon, c.weight_decay, c.clip, at));
+    }
+    // one full training step; shared by tg_train and tg_profile_step
+    void train_step(uint64_t at, float *history_row) {
+        const Config &c = config.base;
+        OP(TG_CLASS_OTHER, tgk_sample_batch(stream, data, data_size, c.seed, at, c.batch, c.context, input, target));
+        forward(input, target, true, nullptr);
+        OP(TG_CLASS_OTHER, tgk_position_means(stream, token_losses, c.batch, c.context, history_row));
+        backward(input);
+        optimize(at);
     }
 
     void read_losses(float *out) { // cuda/runtime.cu:279-290
@@ -322,6 +378,7 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
         e->allocate(e->dqkv, M * 3 * d, false);
         size_t need = tgk_attn_bwd_workspace(c.batch, model->heads, c.context);
         need = std::max(need, tgk_layernorm_bwd_workspace(int(M), int(d)));
+        need = std::max(need, tgk_embed_bwd_workspace(int(M), int(d)));
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(V), int(d)));
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(d), int(F)));
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(F), int(d)));
@@ -477,17 +534,8 @@ TG_API int tg_train(Engine *e, int steps) {
         if (!e->schedule.empty() && e->step + uint64_t(steps) > e->schedule.size())
             throw std::runtime_error("Training would exceed the OneCycle schedule");
         e->use_device();
-        const Config &c = e->config.base;
-        for (int i = 0; i < steps; ++i) {
-            const uint64_t at = e->step + uint64_t(i);
-            ok(tgk_sample_batch(e->stream, e->data, e->data_size, c.seed, at, c.batch, c.context, e->input,
-                                e->target));
-            e->forward(e->input, e->target, true, nullptr);
-            ok(tgk_position_means(e->stream, e->token_losses, c.batch, c.context,
-                                  e->loss_history + size_t(i) * c.context));
-            e->backward(e->input);
-            e->optimize(at);
-        }
+        for (int i = 0; i < steps; ++i)
+            e->train_step(e->step + uint64_t(i), e->loss_history + size_t(i) * e->config.base.context);
         e->last_train_steps = steps;
         e->step += uint64_t(steps);
     });
@@ -578,5 +626,42 @@ TG_API int tg_optimizer_test(Engine *e, const float *gradient, int steps) {
             e->optimize(e->step + uint64_t(i));
         e->step += uint64_t(steps);
         e->sync();
+    });
+}
+
+// Not in the reference.  One training step exactly like tg_train(engine, 1), with a HIP event pair
+// around every operator launch on the engine's stream; returns the summed milliseconds and the
+// number of launches per TG_CLASS_*.  Synchronises.
+TG_API int tg_profile_step(Engine *e, float *class_ms, int *class_launches, int classes) {
+    return guarded([&] {
+        if (!class_ms || !class_launches || classes < TG_CLASSES)
+            throw std::runtime_error("tg_profile_step needs room for TG_CLASSES entries");
+        if (!e->data)
+            throw std::runtime_error("Load data first");
+        if (!e->schedule.empty() && e->step + 1 > e->schedule.size())
+            throw std::runtime_error("Training would exceed the OneCycle schedule");
+        e->use_device();
+        e->profiling = true;
+        try {
+            e->train_step(e->step, e->loss_history);
+        } catch (...) {
+            e->profiling = false;
+            throw;
+        }
+        e->profiling = false;
+        e->last_train_steps = 1;
+        e->step += 1;
+        e->sync();
+        std::fill(class_ms, class_ms + classes, 0.f);
+        std::fill(class_launches, class_launches + classes, 0);
+        for (Engine::Span &span : e->spans) {
+            float ms = 0.f;
+            check_hip(hipEventElapsedTime(&ms, span.start, span.stop));
+            class_ms[span.cls] += ms;
+            class_launches[span.cls] += 1;
+            e->event_pool.push_back(span.start);
+            e->event_pool.push_back(span.stop);
+        }
+        e->spans.clear();
     });
 }
