@@ -278,24 +278,20 @@ int compute_units() {
 struct TileChoice {
     int bm, bn;
 };
-// Cost model: rounds of `cus` concurrent blocks times tile area; small tiles reuse less.
-TileChoice choose_tile(int M, int N, int splits_hint) {
-    const int cus = compute_units();
-    const int candidates[3][2] = {{256, 192}, {256, 256}, {128, 128}};
-    TileChoice best{0, 0};
-    double best_cost = 0;
-    for (auto &c : candidates) {
-        if (M % c[0] || N % c[1])
-            continue;
-        const int64_t tiles = int64_t(M / c[0]) * (N / c[1]) * splits_hint;
-        const int64_t rounds = (tiles + cus - 1) / cus;
-        const double cost = double(rounds) * c[0] * c[1] * (c[0] == 128 ? 1.25 : 1.0);
-        if (!best.bm || cost < best_cost) {
-            best = {c[0], c[1]};
-            best_cost = cost;
-        }
-    }
-    return best;
+// Measured on MI355X at the training shapes (M = 16384, N and K in {768, 2304, 3072}).  The
+// 128x128 tile keeps two blocks resident per CU, so a co-resident block covers the other's
+// prologue, epilogue and global-load latency: it wins whenever the reduction is short (12 k-tiles
+// at K = 768).  With a k-strided operand and a long reduction the 256x192 tile's lower LDS and L2
+// traffic wins instead.
+TileChoice choose_tile(int M, int N, int K, bool kstrided_operand) {
+    const bool big_ok = M % 256 == 0 && N % 192 == 0;
+    if (big_ok && kstrided_operand && K >= 2048)
+        return {256, 192};
+    if (M % 128 == 0 && N % 128 == 0)
+        return {128, 128};
+    if (big_ok)
+        return {256, 192};
+    return {0, 0};
 }
 
 template <int BM, int BN, bool AKC, bool BKC, class Epilogue>
@@ -343,7 +339,7 @@ int wgrad_splits(int tiles, int k_tiles) {
 }
 
 TileChoice wgrad_tile(int rows, int cols) {
-    // few output tiles: the tile choice only needs to divide; prefer the big tiles
+    // few output tiles and a very long reduction: the big tiles win (measured), split-K fills the CUs
     if (rows % 256 == 0 && cols % 192 == 0)
         return {256, 192};
     if (rows % 256 == 0 && cols % 256 == 0)
@@ -361,8 +357,8 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
     return guarded([&] {
         require(M > 0 && N > 0 && K > 0, "gemm_fwd: empty shape");
         require(K % BK == 0, "gemm_fwd: K must be a multiple of 64");
-        const TileChoice tile = choose_tile(M, N, 1);
-        require(tile.bm != 0, "gemm_fwd: M and N must be multiples of 128");
+        const TileChoice tile = choose_tile(M, N, K, false);
+        require(tile.bm != 0, "gemm_fwd: M and N must be multiples of 128 (or of 256 and 192)");
         require(!(residual && gelu_out), "gemm_fwd: residual and GELU epilogues are exclusive");
         check_operand(X, ldx, "X");
         check_operand(W, ldw, "W");
@@ -385,8 +381,8 @@ extern "C" int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uin
     return guarded([&] {
         require(M > 0 && N > 0 && K > 0, "gemm_dgrad: empty shape");
         require(N % BK == 0, "gemm_dgrad: N (the reduced dimension) must be a multiple of 64");
-        const TileChoice tile = choose_tile(M, K, 1);
-        require(tile.bm != 0, "gemm_dgrad: M and K must be multiples of 128");
+        const TileChoice tile = choose_tile(M, K, N, true);
+        require(tile.bm != 0, "gemm_dgrad: M and K must be multiples of 128 (or of 256 and 192)");
         check_operand(dY, lddy, "dY");
         check_operand(W, ldw, "W");
         check_operand(dX, lddx, "dX");
@@ -417,7 +413,7 @@ extern "C" int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uin
         require(M > 0 && N > 0 && K > 0, "gemm_wgrad: empty shape");
         require(M % BK == 0, "gemm_wgrad: M (the reduced dimension) must be a multiple of 64");
         const TileChoice tile = wgrad_tile(N, K);
-        require(tile.bm != 0, "gemm_wgrad: N and K must be multiples of 128");
+        require(tile.bm != 0, "gemm_wgrad: N and K must be multiples of 128 (or of 256 and 192)");
         check_operand(dY, lddy, "dY");
         check_operand(X, ldx, "X");
         require(dW && !(reinterpret_cast<uintptr_t>(dW) & 15) && lddw % 4 == 0,
