@@ -165,6 +165,30 @@ def kernel_sweeps(out):
                       "frac_of_bf16_peak": round(2.5 * flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
 
 
+def traffic_probe():
+    """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: one plain copy of known size (256 MiB in,
+    256 MiB out: the calibration dispatch) followed by one launch of each forward block projection."""
+    import torch
+    from turbogpt_amd.bridge import check, library
+    lib = library()
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.ones(1 << 27, dtype=torch.bfloat16, device="cuda")
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    for k, n in [(768, 2304), (768, 768), (768, 3072), (3072, 768)]:
+        x = torch.randn(M, k, device="cuda").bfloat16()
+        w = torch.randn(n, k, device="cuda").bfloat16()
+        y = torch.empty(M, n, device="cuda", dtype=torch.bfloat16)
+        torch.cuda.synchronize()
+        check(lib.tgk_gemm_fwd(stream, M, n, k, x.data_ptr(), k, w.data_ptr(), k, y.data_ptr(), n, None, 0, None, 0))
+        torch.cuda.synchronize()
+    print(json.dumps({"probe": "traffic", "copy_bytes_each_way": 1 << 28,
+                      "gemm_fwd_algorithmic_bytes": [2 * (M * k + n * k + M * n) for k, n in
+                                                     [(768, 2304), (768, 768), (768, 3072), (3072, 768)]]}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,7 +196,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernels", action="store_true", help="also print the isolated kernel sweeps to stderr")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="run only the copy + forward GEMM dispatches used to read HBM traffic counters")
     args = ap.parse_args()
+    if args.traffic_probe:
+        return traffic_probe()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU (the engine is single-device); run with --gpus 1")
     if not 1 <= args.steps <= 4096 or not 0 <= args.warmup <= 4096:
@@ -211,7 +239,8 @@ def main():
         rate = amount / (per_step_ms * 1e-3) / 1e12 if per_step_ms > 0 else 0.0
         classes[name] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // 3,
                          ("tflops" if kind == "flop" else "tb_per_s"): round(rate, 2)}
-    # dominant MFMA kernel: the forward block-projection GEMM (one template instantiation, 4 launches/layer)
+    # dominant MFMA kernel: the forward block-projection GEMM (one template instantiation, 4 launches/layer);
+    # traffic: profiles/gemm_fwd_hbm_traffic.md (FETCH_SIZE/WRITE_SIZE runs of --traffic-probe), mean of the 4 shapes
     fwd_ms, fwd_launches = profile["gemm_fwd"]
     flops_per_launch = sum(gemm_flops()) / 4
     achieved = flops_per_launch / (fwd_ms / fwd_launches * 1e-3) / 1e12
@@ -233,8 +262,8 @@ def main():
                                "ffn=3072 vocab=256, bf16 weights with fp32 masters, AdamW lr 3e-4 betas 0.9/0.95 "
                                "wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
                    "global_batch": B, "seq_len": T, "parameters": params, "parallelism": "single GPU"},
-        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<256,192,kcontig,kcontig,EpilogueBf16> (forward "
-                     "block projections)", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<128,128,true,true,EpilogueBf16> (forward block "
+                     "projections: QKV, attention-out, MLP-up, MLP-down)", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "flops_per_launch": flops_per_launch,
                      "avg_launch_ms": round(fwd_ms / fwd_launches, 5)},
