@@ -32,7 +32,8 @@ TGK_API const char *tgk_error(void);
  *   residual != NULL : Y = RN_bf16( RN_bf16(acc) + residual )      (bf16 add, cuda/mma.cuh:95-97)
  *   gelu_out != NULL : additionally gelu_out = RN_bf16( gelu(Y) )  (Y keeps the pre-activation;
  *                      stands in for swiglu_activation, cuda/ops.cuh:120-128)
- * M, N multiples of 128, K multiple of 64; pointers 16-byte aligned; ld* multiples of 8. */
+ * M multiple of 128, N multiple of 128 or 192, K multiple of 32; pointers 16-byte aligned; ld*
+ * multiples of 8. */
 TGK_API int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint16_t *X, int ldx,
                  const uint16_t *W, int ldw, uint16_t *Y, int ldy, const uint16_t *residual, int ldr,
                  uint16_t *gelu_out, int ldg);
@@ -42,7 +43,7 @@ TGK_API int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint16_t
  *   dX[M][K] = RN_bf16( dY[M][N] . W[N][K] )
  *   gelu_pre != NULL : dX = RN_bf16( RN_bf16(acc) * gelu'(gelu_pre) )   (fused activation
  *                      backward, stands in for swiglu_backward, cuda/ops.cuh:133-144)
- * M, K multiples of 128, N multiple of 64. */
+ * M multiple of 128, K multiple of 128 or 192, N multiple of 32. */
 TGK_API int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uint16_t *dY, int lddy,
                    const uint16_t *W, int ldw, uint16_t *dX, int lddx, const uint16_t *gelu_pre,
                    int ldu);
@@ -50,7 +51,7 @@ TGK_API int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uint16
 /* Weight gradient, replaces weight_gradient (cuda/ops.cuh:83-109) and, through its fixed-order
  * split-K reduction, reduce_gradients (cuda/trainer.cuh:9-47).
  *   dW[N][K] (= | +=) dY[M][N]^T . X[M][K]      fp32, deterministic
- * N, K multiples of 128, M multiple of 64.  `workspace` must hold
+ * N multiple of 128, K multiple of 128 or 192, M multiple of 32.  `workspace` must hold
  * tgk_gemm_wgrad_workspace(M,N,K) bytes (may be NULL when that is 0). */
 TGK_API int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uint16_t *dY, int lddy,
                    const uint16_t *X, int ldx, float *dW, int lddw, int accumulate, void *workspace,

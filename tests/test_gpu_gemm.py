@@ -114,7 +114,7 @@ def test_rejects_bad_shapes_without_launching():
     t = torch.zeros(256 * 256, dtype=torch.bfloat16, device="cuda")
     p = t.data_ptr()
     assert lib.tgk_gemm_fwd(stream(), 100, 128, 64, p, 64, p, 64, p, 128, None, 0, None, 0) == -1
-    assert b"multiples of 128" in lib.tgk_error()
+    assert b"multiple of 128" in lib.tgk_error()
     assert lib.tgk_gemm_fwd(stream(), 128, 128, 60, p, 64, p, 64, p, 128, None, 0, None, 0) == -1
     assert lib.tgk_gemm_fwd(stream(), 128, 128, 64, p + 2, 64, p, 64, p, 128, None, 0, None, 0) == -1
     assert lib.tgk_gemm_fwd(stream(), 128, 128, 64, None, 64, p, 64, p, 128, None, 0, None, 0) == -1

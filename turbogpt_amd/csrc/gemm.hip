@@ -1,26 +1,29 @@
 // bf16 MFMA GEMM family for gfx950: forward Y = X W^T, dgrad dX = dY W, wgrad dW = dY^T X.
 // Replaces project / matmul+cast_result / weight_gradient of the reference
-// (cuda/mma.cuh:77-108, cuda/ops.cuh:30-55, cuda/ops.cuh:83-109).
+// (cuda/mma.cuh:77-108, cuda/ops.cuh:30-55, cuda/ops.cuh:83-109) and, through the fixed-order
+// split-K fold, reduce_gradients (cuda/trainer.cuh:9-47).
 //
 // One kernel template computes C[m][n] = sum_k A(m,k) B(n,k).  Each operand is either
-// "k-contiguous" (stored [row][k]) or "k-strided" (stored [k][row]); k-strided tiles are
-// transposed in registers on their way into LDS, so the LDS image is always [row][k] and every
-// MFMA fragment is one 16-byte LDS read.
+// "k-contiguous" (stored [row][k]) or "k-strided" (stored [k][row]):
 //   forward : A = X  [M][K] k-contiguous, B = W  [N][K] k-contiguous
-//   dgrad   : A = dY [M][N] k-contiguous, B = W  [N][K] read as (n=K index, k=N index): k-strided
+//   dgrad   : A = dY [M][N] k-contiguous, B = W  [N][K] read as (n = K index, k = N index): k-strided
 //   wgrad   : A = dY [M][N] k-strided (m = out index), B = X [M][K] k-strided, fp32 out, split-K
 //
-// Tile: BM x BN x 64 per 256-thread block, 2x2 waves, v_mfma_f32_32x32x16_bf16 with the operands
-// swapped (instruction A = our B rows) so that a lane ends up holding 4 consecutive n for one m:
-// 8-byte bf16 / 16-byte fp32 stores.  LDS is double buffered, global loads for tile k+1 are in
-// flight while tile k is multiplied; one barrier per k-tile.
+// Data path: global -> LDS directly (global_load_lds_dwordx4: no staging registers, no LDS store
+// instructions), S stages of 32 k deep; the copies run S-1 k-tiles ahead of the MFMAs and keep
+// running across tile boundaries, because a block is persistent and walks a list of work items
+// (tile x split).  LDS tiles are unpadded and XOR-swizzled on 16-byte chunks (a wave-wide copy fills
+// 1 KiB of LDS contiguously, so padding is not available); measured bank conflicts are zero.
+// k-contiguous tiles give each MFMA fragment with one ds_read_b128; k-strided tiles keep the
+// natural [k][row] image and are read with the transposing ds_read_b64_tr_b16.
+// 256 threads = 2x2 waves of v_mfma_f32_32x32x16_bf16; the instruction's A operand is fed with
+// *our B rows* so that a lane ends up holding 4 consecutive n for one m: 8-byte bf16 / 16-byte
+// fp32 stores and a fused epilogue on the fragment.  Fragments of the next k-step are read while
+// the current MFMAs run, also across the per-k-tile barrier.
 #include "common.h"
 #include "../../include/tgk_kernels.h"
 
 namespace {
-
-constexpr int BK = 64;
-constexpr int LDS_STRIDE = BK + 8; // elements; 144-byte rows keep 16-byte reads conflict-free
 
 enum EpilogueMode { EPI_PLAIN = 0, EPI_RESIDUAL = 1, EPI_GELU = 2, EPI_GELU_BWD = 3 };
 
@@ -75,167 +78,241 @@ struct EpilogueF32 {
     }
 };
 
-// Staging of one ROWS x 64 operand tile: global -> registers -> LDS image [row][k].
-// Plain register arrays with compile-time indices only, so they stay in VGPRs.
-template <int ROWS, int NT, bool KCONTIG> struct TileShape {
-    static constexpr int GROUPS = ROWS / 8 * (BK / 4);         // 8-row x 4-k groups (k-strided)
-    static constexpr int GROUP_ITERS = (GROUPS + NT - 1) / NT; // last iteration may be partial
-    static constexpr int CHUNKS = KCONTIG ? ROWS * BK / 8 / NT : GROUP_ITERS * 4; // 16-byte chunks
-    static_assert(!KCONTIG || ROWS * BK / 8 % NT == 0, "tile must divide over the block");
+constexpr int BK = 32;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+// one wave-wide 16-byte-per-lane global -> LDS copy: lane l lands at lds_base + 16*l
+TG_DEVICE void async_copy16(uint32_t lds_base, const void *global) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(global) : "memory");
+}
+template <int N> TG_DEVICE void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// ---- k-contiguous operand tile: ROWS rows x 32 k, 64-byte rows, 16-byte chunk c of row r stored
+// at chunk c ^ ((r >> 2) & 3) ------------------------------------------------------------------
+template <int ROWS> struct TileKC {
+    static constexpr int LOADS = ROWS * 4 / 256; // wave-wide copies per thread per stage
+    static constexpr int BYTES = ROWS * 64;
+    // element offset (relative to the tile origin at k = 0) that this lane fetches for copy j
+    TG_DEVICE static int64_t source_offset(int j, int tid, int ld) {
+        const int wave = tid >> 6, lane = tid & 63;
+        const int row = (j * 4 + wave) * 16 + (lane >> 2), phys = lane & 3;
+        const int chunk = phys ^ ((row >> 2) & 3);
+        return int64_t(row) * ld + chunk * 8;
+    }
+    TG_DEVICE static uint32_t lds_offset(int j, int tid) { // wave-uniform
+        return uint32_t((j * 4 + (tid >> 6)) * 1024);
+    }
+    // fragment for rows row0 + lane%32, k-step ks (16 k): k = ks*16 + 8*(lane/32) .. +7
+    TG_DEVICE static bf16x8 frag(const unsigned char *tile, int row0, int ks, int lane) {
+        const int row = row0 + (lane & 31), chunk = (ks * 2 + (lane >> 5)) ^ ((row >> 2) & 3);
+        return *reinterpret_cast<const bf16x8 *>(tile + row * 64 + chunk * 16);
+    }
 };
 
-template <int ROWS, int NT, bool KCONTIG, int COUNT>
-TG_DEVICE void stage_load(u32x4 (&regs)[COUNT], const bf16_t *base, int ld, int row0, int k0, int tid) {
-    using S = TileShape<ROWS, NT, KCONTIG>;
-    static_assert(COUNT == S::CHUNKS, "register tile size");
-    if constexpr (KCONTIG) {
-#pragma unroll
-        for (int i = 0; i < S::CHUNKS; ++i) {
-            const int c = tid + i * NT, row = c >> 3, kc = c & 7;
-            regs[i] = *reinterpret_cast<const u32x4 *>(base + size_t(row0 + row) * ld + k0 + kc * 8);
-        }
-    } else {
-        // group g: 8 rows (m8) x 4 k (k4); k4 varies fastest over lanes so that the transposed
-        // 8-byte LDS writes of a half wave fall into distinct banks
-#pragma unroll
-        for (int i = 0; i < S::GROUP_ITERS; ++i) {
-            const int g = tid + i * NT, k4 = g & 15, m8 = g >> 4;
-            const bool live = S::GROUPS % NT == 0 || g < S::GROUPS;
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk)
-                regs[i * 4 + kk] = live ? *reinterpret_cast<const u32x4 *>(
-                                              base + size_t(k0 + k4 * 4 + kk) * ld + row0 + m8 * 8)
-                                        : u32x4{0, 0, 0, 0};
-        }
+// ---- k-strided operand tile: source is [k][row]; LDS image 32 k-rows x ROWS columns, natural
+// layout with 16-byte chunk p of k-row r stored at p ^ swizzle(r); read with the transposing load
+template <int ROWS> struct TileKS {
+    static constexpr int LOADS = ROWS * 4 / 256;
+    static constexpr int BYTES = ROWS * 64;
+    static constexpr int CHUNKS_PER_ROW = ROWS / 8;
+    TG_DEVICE static int swizzle(int r) {
+        // row stride of 256 B multiples: 4 consecutive k-rows start in the same bank; 384 B: every other one
+        return ROWS % 128 == 0 ? ((r & 3) << 2) : (((r >> 1) & 1) << 2);
     }
-}
-
-TG_DEVICE void store_transposed_pair(bf16_t *p, uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3) {
-    // r_k holds rows (2j, 2j+1) at k; emit row 2j and row 2j+1 with k = 0..3 contiguous
-    u32x2 even, odd;
-    even.x = (r0 & 0xffffu) | (r1 << 16);
-    even.y = (r2 & 0xffffu) | (r3 << 16);
-    odd.x = (r0 >> 16) | (r1 & 0xffff0000u);
-    odd.y = (r2 >> 16) | (r3 & 0xffff0000u);
-    *reinterpret_cast<u32x2 *>(p) = even;
-    *reinterpret_cast<u32x2 *>(p + LDS_STRIDE) = odd;
-}
-
-template <int ROWS, int NT, bool KCONTIG, int COUNT>
-TG_DEVICE void stage_store(const u32x4 (&regs)[COUNT], bf16_t *lds, int tid) {
-    using S = TileShape<ROWS, NT, KCONTIG>;
-    static_assert(COUNT == S::CHUNKS, "register tile size");
-    if constexpr (KCONTIG) {
-#pragma unroll
-        for (int i = 0; i < S::CHUNKS; ++i) {
-            const int c = tid + i * NT, row = c >> 3, kc = c & 7;
-            *reinterpret_cast<u32x4 *>(lds + row * LDS_STRIDE + kc * 8) = regs[i];
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < S::GROUP_ITERS; ++i) {
-            const int g = tid + i * NT, k4 = g & 15, m8 = g >> 4;
-            if (S::GROUPS % NT == 0 || g < S::GROUPS) {
-                bf16_t *p = lds + (m8 * 8) * LDS_STRIDE + k4 * 4;
-                const u32x4 a = regs[i * 4 + 0], b = regs[i * 4 + 1], c = regs[i * 4 + 2], d = regs[i * 4 + 3];
-                store_transposed_pair(p + 0 * LDS_STRIDE, a.x, b.x, c.x, d.x);
-                store_transposed_pair(p + 2 * LDS_STRIDE, a.y, b.y, c.y, d.y);
-                store_transposed_pair(p + 4 * LDS_STRIDE, a.z, b.z, c.z, d.z);
-                store_transposed_pair(p + 6 * LDS_STRIDE, a.w, b.w, c.w, d.w);
-            }
-        }
+    TG_DEVICE static int64_t source_offset(int j, int tid, int ld) {
+        const int wave = tid >> 6, lane = tid & 63;
+        const int q = (j * 4 + wave) * 64 + lane, r = q / CHUNKS_PER_ROW, p = q - r * CHUNKS_PER_ROW;
+        const int chunk = p ^ swizzle(r);
+        return int64_t(r) * ld + chunk * 8;
     }
+    TG_DEVICE static uint32_t lds_offset(int j, int tid) {
+        return uint32_t((j * 4 + (tid >> 6)) * 1024);
+    }
+    // fragment for columns (operand rows) row0 + lane%32, k = ks*16 + 8*(lane/32) .. +7, natural order
+    TG_DEVICE static bf16x8 frag(const unsigned char *tile, int row0, int ks, int lane) {
+        const int g = lane >> 5, blk = (lane >> 4) & 1, i = lane & 15;
+        const int r = ks * 16 + 8 * g + (i >> 2);
+        const int col = row0 + 16 * blk + 4 * (i & 3);
+        const int chunk = (col >> 3) ^ swizzle(r);
+        const unsigned char *p = tile + r * (ROWS * 2) + chunk * 16 + (i & 1) * 8;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * ROWS * 2));
+        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, both);
+    }
+};
+
+template <int ROWS, bool KC> struct TileOf;
+template <int ROWS> struct TileOf<ROWS, true> { using type = TileKC<ROWS>; };
+template <int ROWS> struct TileOf<ROWS, false> { using type = TileKS<ROWS>; };
+
+template <int BM, int BN, int S> constexpr size_t lds_bytes() {
+    return size_t(S) * (BM + BN) * 64;
 }
 
-template <int BM, int BN> constexpr size_t gemm_lds_bytes() {
-    return size_t(2) * (BM + BN) * LDS_STRIDE * sizeof(bf16_t);
-}
-
-template <int BM, int BN, bool AKC, bool BKC, class Epilogue>
-__global__ __launch_bounds__(256) void gemm_kernel(const bf16_t *__restrict__ A, int lda,
-                                                   const bf16_t *__restrict__ B, int ldb,
-                                                   int k_tiles, int splits, int tiles_n,
-                                                   int tiles_total, Epilogue epilogue) {
-    constexpr int NT = 256, WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+// C[m][n] = sum_k A(m,k) B(n,k).  A k-contiguous: A[m][k] (lda); k-strided: A[k][m] (lda).  Same for B.
+// Work items = tiles x splits, dealt to persistent blocks; loads run S-1 k-tiles ahead of the MFMAs and
+// continue across item boundaries.
+template <int BM, int BN, int S, bool AKC, bool BKC, class Epilogue>
+__global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__ A, int lda,
+                                                    const bf16_t *__restrict__ B, int ldb, int k_tiles,
+                                                    int splits, int tiles_n, int tiles_total,
+                                                    Epilogue epilogue) {
+    using TA = typename TileOf<BM, AKC>::type;
+    using TB = typename TileOf<BN, BKC>::type;
+    constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+    constexpr int LA = TA::LOADS, LB = TB::LOADS, LOADS = LA + LB;
+    constexpr int STAGE = TA::BYTES + TB::BYTES;
     extern __shared__ __align__(16) unsigned char smem[];
-    bf16_t *const sA = reinterpret_cast<bf16_t *>(smem);    // two stages of BM rows
-    bf16_t *const sB = sA + 2 * BM * LDS_STRIDE;             // two stages of BN rows
-
-    // Blocks are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of tiles so
-    // that tiles sharing operand rows meet in the same L2.
-    const int blocks = gridDim.x;
-    int logical = blockIdx.x;
-    if ((blocks & 7) == 0)
-        logical = (logical & 7) * (blocks >> 3) + (logical >> 3);
-    const int split = logical / tiles_total, tile = logical - split * tiles_total;
-    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
-    const int kt0 = int(int64_t(split) * k_tiles / splits);
-    const int kt1 = int(int64_t(split + 1) * k_tiles / splits);
+    const uint32_t smem_base = uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
-    const int frag_row = lane & 31, frag_k = (lane >> 5) * 8;
+    const int items = tiles_total * splits, stride = gridDim.x;
 
-    f32x16 acc[FM][FN];
+    // item -> (m0, n0, first k-tile, k-tile count); blocks of one XCD get contiguous tiles
+    auto locate = [&](int item, int &m0, int &n0, int &kt0, int &nk) {
+        int logical = item;
+        if ((items & 7) == 0)
+            logical = (item & 7) * (items >> 3) + (item >> 3);
+        const int split = logical / tiles_total, tile = logical - split * tiles_total;
+        m0 = (tile / tiles_n) * BM;
+        n0 = (tile % tiles_n) * BN;
+        kt0 = split * k_tiles / splits;
+        nk = (split + 1) * k_tiles / splits - kt0;
+        return split;
+    };
+
+    // ---- producer state -------------------------------------------------------------------------
+    int p_item = blockIdx.x, p_left = 0, p_slot = 0;
+    const bf16_t *pa[LA], *pb[LB];
+    int64_t a_step = AKC ? BK : int64_t(BK) * lda, b_step = BKC ? BK : int64_t(BK) * ldb;
+    auto producer_open = [&]() { // point the copy sources at the first k-tile of p_item
+        int m0, n0, kt0, nk;
+        locate(p_item, m0, n0, kt0, nk);
+        p_left = nk;
+        const bf16_t *a0 = AKC ? A + int64_t(m0) * lda + int64_t(kt0) * BK : A + int64_t(kt0) * BK * lda + m0;
+        const bf16_t *b0 = BKC ? B + int64_t(n0) * ldb + int64_t(kt0) * BK : B + int64_t(kt0) * BK * ldb + n0;
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+        for (int j = 0; j < LA; ++j)
+            pa[j] = a0 + TA::source_offset(j, tid, lda);
+#pragma unroll
+        for (int j = 0; j < LB; ++j)
+            pb[j] = b0 + TB::source_offset(j, tid, ldb);
+    };
+    auto produce = [&]() { // issue the copies of one k-tile into slot p_slot; returns false when out of work
+        if (p_left == 0) {
+            p_item += stride;
+            if (p_item >= items)
+                return false;
+            producer_open();
+        }
+        const uint32_t base = smem_base + uint32_t(p_slot) * STAGE;
+#pragma unroll
+        for (int j = 0; j < LA; ++j) {
+            async_copy16(__builtin_amdgcn_readfirstlane(base + TA::lds_offset(j, tid)), pa[j]);
+            pa[j] += a_step;
+        }
+#pragma unroll
+        for (int j = 0; j < LB; ++j) {
+            async_copy16(__builtin_amdgcn_readfirstlane(base + TA::BYTES + TB::lds_offset(j, tid)), pb[j]);
+            pb[j] += b_step;
+        }
+        --p_left;
+        p_slot = p_slot + 1 == S ? 0 : p_slot + 1;
+        return true;
+    };
+
+    if (p_item >= items)
+        return;
+    producer_open();
+    int inflight = 0; // stages issued and not yet consumed
+#pragma unroll
+    for (int s = 0; s < S - 1; ++s)
+        if (produce())
+            ++inflight;
+
+    // Wait until at most `allowed` of this wave's newest stages are still in flight.
+    auto wait_stages = [&](int allowed) {
+        if (S >= 5 && allowed >= 3)
+            wait_vmcnt<3 * LOADS>();
+        else if (S >= 4 && allowed == 2)
+            wait_vmcnt<2 * LOADS>();
+        else if (S >= 3 && allowed == 1)
+            wait_vmcnt<1 * LOADS>();
+        else
+            wait_vmcnt<0>();
+    };
+    auto load_frags = [&](bf16x8 (&af)[FM], bf16x8 (&bfr)[FN], int slot, int ks) {
+        const unsigned char *sa = smem + slot * STAGE, *sb = sa + TA::BYTES;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+            af[i] = TA::frag(sa, wm + i * 32, ks, lane);
 #pragma unroll
         for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                acc[i][j][r] = 0.f;
+            bfr[j] = TB::frag(sb, wn + j * 32, ks, lane);
+    };
 
-    u32x4 regsA[TileShape<BM, NT, AKC>::CHUNKS], regsB[TileShape<BN, NT, BKC>::CHUNKS];
-    if (kt0 < kt1) {
-        stage_load<BM, NT, AKC>(regsA, A, lda, m0, kt0 * BK, tid);
-        stage_load<BN, NT, BKC>(regsB, B, ldb, n0, kt0 * BK, tid);
-        stage_store<BM, NT, AKC>(regsA, sA, tid);
-        stage_store<BN, NT, BKC>(regsB, sB, tid);
-    }
+    // ---- consumer ---------------------------------------------------------------------------------
+    // Stages are made visible one k-tile early: iteration t starts by making stage t+1 visible, so the
+    // first fragments of tile t+1 can be read at the end of iteration t and the MFMAs of the next
+    // iteration start straight after its barrier.
+    bf16x8 af0[FM], bf0[FN], af1[FM], bf1[FN];
+    int c_slot = 0;
+    wait_stages(inflight - 1); // stage 0 landed
     __syncthreads();
-    for (int kt = kt0; kt < kt1; ++kt) {
-        const int cur = (kt - kt0) & 1;
-        const bool more = kt + 1 < kt1;
-        if (more) {
-            stage_load<BM, NT, AKC>(regsA, A, lda, m0, (kt + 1) * BK, tid);
-            stage_load<BN, NT, BKC>(regsB, B, ldb, n0, (kt + 1) * BK, tid);
-        }
-        const bf16_t *a_base = sA + cur * (BM * LDS_STRIDE) + (wm + frag_row) * LDS_STRIDE + frag_k;
-        const bf16_t *b_base = sB + cur * (BN * LDS_STRIDE) + (wn + frag_row) * LDS_STRIDE + frag_k;
+    load_frags(af0, bf0, 0, 0);
+    for (int item = blockIdx.x; item < items; item += stride) {
+        int m0, n0, kt0, nk;
+        const int split = locate(item, m0, n0, kt0, nk);
+        f32x16 acc[FM][FN];
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 af[FM], bfr[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-                af[i] = *reinterpret_cast<const bf16x8 *>(a_base + i * 32 * LDS_STRIDE + ks * 16);
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
             for (int j = 0; j < FN; ++j)
-                bfr[j] = *reinterpret_cast<const bf16x8 *>(b_base + j * 32 * LDS_STRIDE + ks * 16);
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[i][j][r] = 0.f;
+        for (int kt = 0; kt < nk; ++kt) {
+            // in flight now: the stage being consumed (landed), then inflight-1 younger ones; the next one
+            // must land too
+            wait_stages(inflight >= 2 ? inflight - 2 : 0);
+            __syncthreads();
+            --inflight;
+            if (produce())
+                ++inflight;
+            const int next_slot = c_slot + 1 == S ? 0 : c_slot + 1;
+            load_frags(af1, bf1, c_slot, 1);
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf0[j], af0[i], acc[i][j], 0, 0, 0);
+            load_frags(af0, bf0, next_slot, 0);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[j], af1[i], acc[i][j], 0, 0, 0);
+            c_slot = next_slot;
         }
-        if (more) {
-            stage_store<BM, NT, AKC>(regsA, sA + (cur ^ 1) * (BM * LDS_STRIDE), tid);
-            stage_store<BN, NT, BKC>(regsB, sB + (cur ^ 1) * (BN * LDS_STRIDE), tid);
-        }
-        __syncthreads();
+        const int out_m = m0 + wm + (lane & 31), out_n = n0 + wn + (lane >> 5) * 4;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                                        acc[i][j][q * 4 + 3]};
+                    epilogue(out_m + i * 32, out_n + j * 32 + q * 8, v, split);
+                }
     }
-
-    // accumulator register r of a lane: m = lane%32, n = 8*(r/4) + 4*(lane/32) + r%4
-    const int out_m = m0 + wm + frag_row, out_n = n0 + wn + (lane >> 5) * 4;
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
-                                    acc[i][j][q * 4 + 3]};
-                epilogue(out_m + i * 32, out_n + j * 32 + q * 8, v, split);
-            }
+    wait_vmcnt<0>();
 }
 
 // Sums split-K slabs in a fixed order (deterministic) into the fp32 gradient.
@@ -275,30 +352,28 @@ int compute_units() {
     return cached;
 }
 
-struct TileChoice {
-    int bm, bn;
-};
-// Measured on MI355X at the training shapes (M = 16384, N and K in {768, 2304, 3072}).  The
-// 128x128 tile keeps two blocks resident per CU, so a co-resident block covers the other's
-// prologue, epilogue and global-load latency: it wins whenever the reduction is short (12 k-tiles
-// at K = 768).  With a k-strided operand and a long reduction the 256x192 tile's lower LDS and L2
-// traffic wins instead.
-TileChoice choose_tile(int M, int N, int K, bool kstrided_operand) {
-    const bool big_ok = M % 256 == 0 && N % 192 == 0;
-    if (big_ok && kstrided_operand && K >= 2048)
-        return {256, 192};
-    if (M % 128 == 0 && N % 128 == 0)
-        return {128, 128};
-    if (big_ok)
-        return {256, 192};
-    return {0, 0};
+enum Tile { TILE_NONE, TILE_128x128, TILE_128x192 };
+// 128x192, 3 stages (60 KiB of LDS, <= 186 VGPRs): two blocks are resident per CU, so one block's
+// MFMAs cover the other's epilogue, barrier and copy-issue gaps; at N = 768 / 2304 / 3072 and
+// M = 16384 it gives 512 / 1536 / 2048 tiles, whole multiples of the 512 resident blocks.  Measured
+// on MI355X it beats a 256x192 single-block-per-CU variant on every training shape.
+// 128x128, 4 stages: shapes that 192 does not divide.
+Tile choose_tile(int rows, int cols) {
+    if (rows % 128 == 0 && cols % 192 == 0)
+        return TILE_128x192;
+    if (rows % 128 == 0 && cols % 128 == 0)
+        return TILE_128x128;
+    return TILE_NONE;
 }
+int tile_rows(Tile) { return 128; }
+int tile_cols(Tile t) { return t == TILE_128x128 ? 128 : 192; }
+int resident_blocks(Tile) { return compute_units() * 2; }
 
-template <int BM, int BN, bool AKC, bool BKC, class Epilogue>
+template <int BM, int BN, int S, bool AKC, bool BKC, class Epilogue>
 void launch_gemm(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N,
-                 int K, int splits, const Epilogue &epilogue) {
-    auto kernel = gemm_kernel<BM, BN, AKC, BKC, Epilogue>;
-    constexpr size_t lds = gemm_lds_bytes<BM, BN>();
+                 int K, int splits, int max_blocks, const Epilogue &epilogue) {
+    auto kernel = gemm_kernel<BM, BN, S, AKC, BKC, Epilogue>;
+    constexpr size_t lds = lds_bytes<BM, BN, S>();
     static bool configured = false;
     if (!configured) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -306,21 +381,20 @@ void launch_gemm(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, 
                   "gemm LDS size: ");
         configured = true;
     }
-    const int tiles_n = N / BN, tiles = (M / BM) * tiles_n;
-    hipLaunchKernelGGL(kernel, dim3(tiles * splits), dim3(256), lds, stream, A, lda, B, ldb, K / BK,
-                       splits, tiles_n, tiles, epilogue);
+    const int tiles_n = N / BN, tiles = (M / BM) * tiles_n, items = tiles * splits;
+    hipLaunchKernelGGL(kernel, dim3(items < max_blocks ? items : max_blocks), dim3(256), lds, stream, A, lda, B,
+                       ldb, K / BK, splits, tiles_n, tiles, epilogue);
     check_hip(hipGetLastError(), "gemm launch: ");
 }
 
 template <bool AKC, bool BKC, class Epilogue>
-void dispatch_gemm(hipStream_t stream, TileChoice tile, const bf16_t *A, int lda, const bf16_t *B,
-                   int ldb, int M, int N, int K, int splits, const Epilogue &epilogue) {
-    if (tile.bm == 256 && tile.bn == 192)
-        launch_gemm<256, 192, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
-    else if (tile.bm == 256 && tile.bn == 256)
-        launch_gemm<256, 256, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
+void dispatch_gemm(hipStream_t stream, Tile tile, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M,
+                   int N, int K, int splits, const Epilogue &epilogue) {
+    const int blocks = resident_blocks(tile);
+    if (tile == TILE_128x192)
+        launch_gemm<128, 192, 3, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, blocks, epilogue);
     else
-        launch_gemm<128, 128, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
+        launch_gemm<128, 128, 4, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, blocks, epilogue);
 }
 
 void check_operand(const void *p, int ld, const char *name) {
@@ -329,24 +403,13 @@ void check_operand(const void *p, int ld, const char *name) {
                                     " must be non-null, 16-byte aligned, leading dimension % 8 == 0");
 }
 
-int wgrad_splits(int tiles, int k_tiles) {
-    const int cus = compute_units();
-    int splits = cus / tiles;
+// wgrad has few output tiles and a very long reduction: split it so the work items fill the GPU
+int wgrad_splits(Tile tile, int tiles, int k_tiles) {
+    int splits = resident_blocks(tile) / tiles;
     if (splits < 1)
         splits = 1;
-    const int max_by_k = k_tiles / 4 > 0 ? k_tiles / 4 : 1; // at least 4 k-tiles per split
+    const int max_by_k = k_tiles / 8 > 0 ? k_tiles / 8 : 1; // at least 8 k-tiles (256 tokens) per split
     return splits < max_by_k ? splits : max_by_k;
-}
-
-TileChoice wgrad_tile(int rows, int cols) {
-    // few output tiles and a very long reduction: the big tiles win (measured), split-K fills the CUs
-    if (rows % 256 == 0 && cols % 192 == 0)
-        return {256, 192};
-    if (rows % 256 == 0 && cols % 256 == 0)
-        return {256, 256};
-    if (rows % 128 == 0 && cols % 128 == 0)
-        return {128, 128};
-    return {0, 0};
 }
 
 } // namespace
@@ -356,9 +419,9 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
                             const uint16_t *residual, int ldr, uint16_t *gelu_out, int ldg) {
     return guarded([&] {
         require(M > 0 && N > 0 && K > 0, "gemm_fwd: empty shape");
-        require(K % BK == 0, "gemm_fwd: K must be a multiple of 64");
-        const TileChoice tile = choose_tile(M, N, K, false);
-        require(tile.bm != 0, "gemm_fwd: M and N must be multiples of 128 (or of 256 and 192)");
+        require(K % BK == 0, "gemm_fwd: K must be a multiple of 32");
+        const Tile tile = choose_tile(M, N);
+        require(tile != TILE_NONE, "gemm_fwd: M must be a multiple of 128 and N of 128 or 192");
         require(!(residual && gelu_out), "gemm_fwd: residual and GELU epilogues are exclusive");
         check_operand(X, ldx, "X");
         check_operand(W, ldw, "W");
@@ -380,9 +443,9 @@ extern "C" int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uin
                               const uint16_t *gelu_pre, int ldu) {
     return guarded([&] {
         require(M > 0 && N > 0 && K > 0, "gemm_dgrad: empty shape");
-        require(N % BK == 0, "gemm_dgrad: N (the reduced dimension) must be a multiple of 64");
-        const TileChoice tile = choose_tile(M, K, N, true);
-        require(tile.bm != 0, "gemm_dgrad: M and K must be multiples of 128 (or of 256 and 192)");
+        require(N % BK == 0, "gemm_dgrad: N (the reduced dimension) must be a multiple of 32");
+        const Tile tile = choose_tile(M, K);
+        require(tile != TILE_NONE, "gemm_dgrad: M must be a multiple of 128 and K of 128 or 192");
         check_operand(dY, lddy, "dY");
         check_operand(W, ldw, "W");
         check_operand(dX, lddx, "dX");
@@ -399,10 +462,10 @@ extern "C" int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uin
 extern "C" size_t tgk_gemm_wgrad_workspace(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0 || M % BK)
         return 0;
-    const TileChoice tile = wgrad_tile(N, K);
-    if (!tile.bm)
+    const Tile tile = choose_tile(N, K);
+    if (tile == TILE_NONE)
         return 0;
-    const int splits = wgrad_splits((N / tile.bm) * (K / tile.bn), M / BK);
+    const int splits = wgrad_splits(tile, (N / tile_rows(tile)) * (K / tile_cols(tile)), M / BK);
     return splits > 1 ? size_t(splits) * N * K * sizeof(float) : 0;
 }
 
@@ -411,14 +474,14 @@ extern "C" int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uin
                               void *workspace, size_t workspace_bytes) {
     return guarded([&] {
         require(M > 0 && N > 0 && K > 0, "gemm_wgrad: empty shape");
-        require(M % BK == 0, "gemm_wgrad: M (the reduced dimension) must be a multiple of 64");
-        const TileChoice tile = wgrad_tile(N, K);
-        require(tile.bm != 0, "gemm_wgrad: N and K must be multiples of 128 (or of 256 and 192)");
+        require(M % BK == 0, "gemm_wgrad: M (the reduced dimension) must be a multiple of 32");
+        const Tile tile = choose_tile(N, K);
+        require(tile != TILE_NONE, "gemm_wgrad: N must be a multiple of 128 and K of 128 or 192");
         check_operand(dY, lddy, "dY");
         check_operand(X, ldx, "X");
         require(dW && !(reinterpret_cast<uintptr_t>(dW) & 15) && lddw % 4 == 0,
                 "gemm_wgrad: dW must be 16-byte aligned with leading dimension % 4 == 0");
-        const int splits = wgrad_splits((N / tile.bm) * (K / tile.bn), M / BK);
+        const int splits = wgrad_splits(tile, (N / tile_rows(tile)) * (K / tile_cols(tile)), M / BK);
         if (splits == 1) {
             EpilogueF32 e{dW, lddw, 0, accumulate};
             dispatch_gemm<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, 1, e);
