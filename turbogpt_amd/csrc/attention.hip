@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *__restric
 // Scores are produced as S[query][key] here: one lane owns one KEY, which is the row index of
 // both outputs.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
+__global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
     const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
     const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ LSE,
     const float *__restrict__ delta, bf16_t *__restrict__ dK, bf16_t *__restrict__ dV, int lddq, int T,
@@ -264,41 +264,43 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(
             tile_load(qr, qbase + size_t(q0 + 64) * ld, ld, tid);
             tile_load(gr, gbase + size_t(q0 + 64) * lddo, lddo, tid);
         }
-        if (q0 + 63 >= wave_k0) { // some query of this tile sees this wave's keys (wave uniform)
-            f32x16 s[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
+        // the two 32-query halves of the tile are processed one after the other to keep the live
+        // accumulators (and with them the register count, hence two resident blocks per CU) down
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
+        for (int qt = 0; qt < 2; ++qt) {
+            const int qh = q0 + qt * 32;
+            if (qh + 31 < wave_k0) // every query of this half precedes this wave's keys (wave uniform)
+                continue;
+            f32x16 s = zero16(), dp = zero16();
 #pragma unroll
-                for (int qt = 0; qt < 2; ++qt) {
-                    s[qt] = mfma(frag_rows(sQ[cur], qt * 32, ks * 16, lane), kf[ks], s[qt]);
-                    dp[qt] = mfma(frag_rows(sdO[cur], qt * 32, ks * 16, lane), vf[ks], dp[qt]);
+            for (int ks = 0; ks < 4; ++ks) {
+                s = mfma(frag_rows(sQ[cur], qt * 32, ks * 16, lane), kf[ks], s);
+                dp = mfma(frag_rows(sdO[cur], qt * 32, ks * 16, lane), vf[ks], dp);
+            }
+            const bool diagonal = qh < wave_k0 + 31;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int q = qh + 8 * q4 + 4 * g;
+                const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_row + q);
+                const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_row + q);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = q4 * 4 + e;
+                    float p = exp2_fast(fmaf(s[r], c, -lse4[e] * LOG2E));
+                    if (diagonal && krow > q + e)
+                        p = 0.f;
+                    s[r] = p;
+                    dp[r] = p * (dp[r] - del4[e]);
                 }
-            const bool diagonal = q0 < wave_k0 + 31;
+            }
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) {
-                    const int q = q0 + qt * 32 + 8 * q4 + 4 * g;
-                    const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_row + q);
-                    const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_row + q);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int r = q4 * 4 + e;
-                        float p = exp2_fast(fmaf(s[qt][r], c, -lse4[e] * LOG2E));
-                        if (diagonal && krow > q + e)
-                            p = 0.f;
-                        s[qt][r] = p;
-                        dp[qt][r] = p * (dp[qt][r] - del4[e]);
-                    }
-                }
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                const bf16x8 pf = acc_to_frag(s[kk >> 1], kk & 1);
-                const bf16x8 dsf = acc_to_frag(dp[kk >> 1], kk & 1);
+            for (int kk2 = 0; kk2 < 2; ++kk2) {
+                const bf16x8 pf = acc_to_frag(s, kk2);
+                const bf16x8 dsf = acc_to_frag(dp, kk2);
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt) {
-                    dv[dt] = mfma(frag_cols(sdO[cur], kk * 16, dt * 32, lane), pf, dv[dt]);
-                    dk[dt] = mfma(frag_cols(sQ[cur], kk * 16, dt * 32, lane), dsf, dk[dt]);
+                    dv[dt] = mfma(frag_cols(sdO[cur], qt * 32 + kk2 * 16, dt * 32, lane), pf, dv[dt]);
+                    dk[dt] = mfma(frag_cols(sQ[cur], qt * 32 + kk2 * 16, dt * 32, lane), dsf, dk[dt]);
                 }
             }
         }
