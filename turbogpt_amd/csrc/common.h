@@ -36,13 +36,31 @@ TG_DEVICE float bf16_hi(uint32_t pair) {
 TG_DEVICE float round_bf16(float f) {
     return bf16_to_float(float_to_bf16(f));
 }
-// exact-erf GELU and its derivative
+// GELU with the exact-erf definition and its derivative.  erf is evaluated with Abramowitz-Stegun
+// 7.1.26 (|error| <= 1.5e-7, far below bf16 resolution): one reciprocal, one exp2 and a degree-5
+// Horner chain, branch free.  gelu'(x) = Phi(x) + x phi(x) shares the exponential, because
+// erf(x/sqrt2) needs exp(-x^2/2) and so does phi.
+struct GeluParts {
+    float cdf; // Phi(x) = 0.5 (1 + erf(x / sqrt 2))
+    float pdf; // phi(x) = exp(-x^2 / 2) / sqrt(2 pi)
+};
+TG_DEVICE GeluParts gelu_parts(float x) {
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    const float e = __builtin_amdgcn_exp2f(x * x * -0.72134752044448170f); // exp(-x^2/2)
+    float poly = fmaf(1.061405429f, t, -1.453152027f);
+    poly = fmaf(poly, t, 1.421413741f);
+    poly = fmaf(poly, t, -0.284496736f);
+    poly = fmaf(poly, t, 0.254829592f);
+    const float tail = 0.5f * poly * t * e; // 0.5 erfc(|x|/sqrt2)
+    return {x < 0.f ? tail : 1.0f - tail, 0.39894228040143268f * e};
+}
 TG_DEVICE float gelu_f(float x) {
-    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+    return x * gelu_parts(x).cdf;
 }
 TG_DEVICE float gelu_grad_f(float x) {
-    return 0.5f * (1.0f + erff(x * 0.70710678118654752f)) +
-           x * 0.39894228040143268f * __expf(-0.5f * x * x);
+    const GeluParts g = gelu_parts(x);
+    return fmaf(x, g.pdf, g.cdf);
 }
 TG_DEVICE float wave_sum(float x) {
 #pragma unroll

@@ -106,7 +106,9 @@ __global__ __launch_bounds__(256) void embed_bwd_positions_kernel(const bf16_t *
 }
 
 // ---- LayerNorm --------------------------------------------------------------------------------
-// One wave per row, the row lives in registers (two-pass mean / variance).
+// One wave per row, the row lives in registers (two-pass mean / variance).  NC = 16-byte chunks per
+// lane (D <= NC * 512): sizing the register tile to the row keeps occupancy up on narrow models.
+template <int NC>
 __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__restrict__ x,
                                                             const uint16_t *__restrict__ gamma_hi,
                                                             const uint16_t *__restrict__ gamma_lo,
@@ -117,10 +119,10 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, chunks = D >> 3;
     const float inv_d = 1.0f / D;
     for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
-        float v[MAX_LN_CHUNKS][8];
+        float v[NC][8];
         float sum = 0.f;
 #pragma unroll
-        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+        for (int j = 0; j < NC; ++j) {
             const int c = lane + j * 64;
             if (c < chunks) {
                 unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
         const float mean = wave_sum(sum) * inv_d;
         float sq = 0.f;
 #pragma unroll
-        for (int j = 0; j < MAX_LN_CHUNKS; ++j)
+        for (int j = 0; j < NC; ++j)
             if (lane + j * 64 < chunks)
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
                 }
         const float inv = 1.0f / sqrtf(wave_sum(sq) * inv_d + eps);
 #pragma unroll
-        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+        for (int j = 0; j < NC; ++j) {
             const int c = lane + j * 64;
             if (c < chunks) {
                 float gm[8], bt[8], o[8];
@@ -157,6 +159,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
 }
 
 // dx (+ residual), and per-block partial sums of dgamma / dbeta into partial[block][2][D].
+template <int NC>
 __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__restrict__ x,
                                                             const bf16_t *__restrict__ dy,
                                                             const uint16_t *__restrict__ gamma_hi,
@@ -167,9 +170,9 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
     extern __shared__ float lds[]; // [4 waves][2][D]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, chunks = D >> 3;
     const float inv_d = 1.0f / D;
-    float dg[MAX_LN_CHUNKS][8], db[MAX_LN_CHUNKS][8], gm[MAX_LN_CHUNKS][8];
+    float dg[NC][8], db[NC][8], gm[NC][8];
 #pragma unroll
-    for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+    for (int j = 0; j < NC; ++j) {
         const int c = lane + j * 64;
 #pragma unroll
         for (int k = 0; k < 8; ++k)
@@ -178,10 +181,10 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
             join8(gamma_hi + c * 8, gamma_lo + c * 8, gm[j]);
     }
     for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
-        float v[MAX_LN_CHUNKS][8], g[MAX_LN_CHUNKS][8];
+        float v[NC][8], g[NC][8];
         float sum = 0.f;
 #pragma unroll
-        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+        for (int j = 0; j < NC; ++j) {
             const int c = lane + j * 64;
             if (c < chunks) {
                 unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
         const float mean = wave_sum(sum) * inv_d;
         float sq = 0.f;
 #pragma unroll
-        for (int j = 0; j < MAX_LN_CHUNKS; ++j)
+        for (int j = 0; j < NC; ++j)
             if (lane + j * 64 < chunks)
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
@@ -204,7 +207,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
         const float inv = 1.0f / sqrtf(wave_sum(sq) * inv_d + eps);
         float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-        for (int j = 0; j < MAX_LN_CHUNKS; ++j)
+        for (int j = 0; j < NC; ++j)
             if (lane + j * 64 < chunks)
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
@@ -218,7 +221,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
         s1 = wave_sum(s1) * inv_d;
         s2 = wave_sum(s2) * inv_d;
 #pragma unroll
-        for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+        for (int j = 0; j < NC; ++j) {
             const int c = lane + j * 64;
             if (c < chunks) {
                 float o[8];
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
     }
     float *mine = lds + wave * 2 * D;
 #pragma unroll
-    for (int j = 0; j < MAX_LN_CHUNKS; ++j) {
+    for (int j = 0; j < NC; ++j) {
         const int c = lane + j * 64;
         if (c < chunks)
 #pragma unroll
@@ -254,29 +257,35 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
         partial[size_t(blockIdx.x) * 2 * D + i] =
             (lds[i] + lds[2 * D + i]) + (lds[4 * D + i] + lds[6 * D + i]);
 }
-// dgamma[c] (+)= sum_b partial[b][0][c], dbeta likewise.  64 columns per block, 4 interleaved
-// block phases per column combined in a fixed order.
+// dgamma[c] (+)= sum_b partial[b][0][c], dbeta likewise.  16 columns x 16 row phases per block; every
+// thread keeps 8 independent loads in flight; phases are combined in a fixed order.
 __global__ __launch_bounds__(256) void layernorm_bwd_reduce_kernel(const float *__restrict__ partial,
                                                                    int blocks, int D,
                                                                    float *__restrict__ dgamma,
                                                                    float *__restrict__ dbeta,
                                                                    int accumulate) {
-    __shared__ float part[4][64];
-    const int col = threadIdx.x & 63, phase = threadIdx.x >> 6, i = blockIdx.x * 64 + col;
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    __shared__ float part[16][17];
+    const int col = threadIdx.x & 15, phase = threadIdx.x >> 4, i = blockIdx.x * 16 + col;
+    const size_t row_stride = size_t(2) * D;
+    float s[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        s[u] = 0.f;
     int b = phase;
-    for (; b + 12 < blocks; b += 16) { // four independent loads in flight per thread
-        s0 += partial[size_t(b) * 2 * D + i];
-        s1 += partial[size_t(b + 4) * 2 * D + i];
-        s2 += partial[size_t(b + 8) * 2 * D + i];
-        s3 += partial[size_t(b + 12) * 2 * D + i];
+    for (; b + 16 * 7 < blocks; b += 16 * 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            s[u] += partial[size_t(b + 16 * u) * row_stride + i];
     }
-    for (; b < blocks; b += 4)
-        s0 += partial[size_t(b) * 2 * D + i];
-    part[phase][col] = (s0 + s1) + (s2 + s3);
+    for (; b < blocks; b += 16)
+        s[0] += partial[size_t(b) * row_stride + i];
+    part[phase][col] = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
     __syncthreads();
     if (phase == 0) {
-        const float sum = (part[0][col] + part[1][col]) + (part[2][col] + part[3][col]);
+        float sum = 0.f;
+#pragma unroll
+        for (int p = 0; p < 16; ++p)
+            sum += part[p][col];
         float *out = i < D ? dgamma + i : dbeta + (i - D);
         *out = accumulate ? *out + sum : sum;
     }
@@ -507,14 +516,22 @@ extern "C" int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint
         aligned(gamma_lo, "layernorm: gamma_lo");
         aligned(beta_hi, "layernorm: beta_hi");
         aligned(beta_lo, "layernorm: beta_lo");
-        hipLaunchKernelGGL(layernorm_fwd_kernel, dim3(grid_for(rows, 4, 8192)), dim3(256), 0, stream, x, gamma_hi,
-                           gamma_lo, beta_hi, beta_lo, y, rows, D, eps);
+        const dim3 grid(grid_for(rows, 4, 8192));
+        if (D <= 512)
+            hipLaunchKernelGGL(layernorm_fwd_kernel<1>, grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo, beta_hi,
+                               beta_lo, y, rows, D, eps);
+        else if (D <= 1024)
+            hipLaunchKernelGGL(layernorm_fwd_kernel<2>, grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo, beta_hi,
+                               beta_lo, y, rows, D, eps);
+        else
+            hipLaunchKernelGGL(layernorm_fwd_kernel<4>, grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo, beta_hi,
+                               beta_lo, y, rows, D, eps);
         check_hip(hipGetLastError(), "layernorm_fwd launch: ");
     });
 }
 
 static int layernorm_bwd_blocks(int rows) {
-    return grid_for(rows, 16, 512);
+    return grid_for(rows, 8, 1024);
 }
 extern "C" size_t tgk_layernorm_bwd_workspace(int rows, int D) {
     return rows > 0 && D > 0 ? size_t(layernorm_bwd_blocks(rows)) * 2 * D * sizeof(float) : 0;
@@ -536,9 +553,17 @@ extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint
                 "layernorm_bwd: workspace too small (see tgk_layernorm_bwd_workspace)");
         const int blocks = layernorm_bwd_blocks(rows);
         float *partial = static_cast<float *>(workspace);
-        hipLaunchKernelGGL(layernorm_bwd_kernel, dim3(blocks), dim3(256), size_t(8) * D * sizeof(float), stream, x,
-                           dy, gamma_hi, gamma_lo, dx, partial, rows, D, eps, residual);
-        hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3(2 * D / 64), dim3(256), 0, stream, partial, blocks, D,
+        const size_t lds = size_t(8) * D * sizeof(float);
+        if (D <= 512)
+            hipLaunchKernelGGL(layernorm_bwd_kernel<1>, dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,
+                               gamma_lo, dx, partial, rows, D, eps, residual);
+        else if (D <= 1024)
+            hipLaunchKernelGGL(layernorm_bwd_kernel<2>, dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,
+                               gamma_lo, dx, partial, rows, D, eps, residual);
+        else
+            hipLaunchKernelGGL(layernorm_bwd_kernel<4>, dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,
+                               gamma_lo, dx, partial, rows, D, eps, residual);
+        hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3(2 * D / 16), dim3(256), 0, stream, partial, blocks, D,
                            dgamma, dbeta, accumulate);
         check_hip(hipGetLastError(), "layernorm_bwd launch: ");
     });
