@@ -27,7 +27,11 @@ namespace {
 
 enum EpilogueMode { EPI_PLAIN = 0, EPI_RESIDUAL = 1, EPI_GELU = 2, EPI_GELU_BWD = 3 };
 
+// Epilogues work on 4 consecutive n of one m.  An epilogue that needs a second input (residual,
+// saved pre-activation) declares AUX: the kernel fetches those 8 bytes two k-tiles before the end
+// of the reduction, so the epilogue does not wait on memory.
 struct EpilogueBf16 {
+    static constexpr bool AUX = true;
     bf16_t *out;
     int ld_out;
     const bf16_t *aux; // residual (EPI_RESIDUAL) or saved pre-activation (EPI_GELU_BWD)
@@ -35,21 +39,22 @@ struct EpilogueBf16 {
     bf16_t *out2; // GELU output (EPI_GELU)
     int ld_out2;
     int mode;
-    int split_stride_unused;
-    TG_DEVICE void operator()(int m, int n, const float (&v)[4], int) const {
+    TG_DEVICE bool wants_aux() const { return mode == EPI_RESIDUAL || mode == EPI_GELU_BWD; }
+    TG_DEVICE u32x2 load_aux(int m, int n) const {
+        return *reinterpret_cast<const u32x2 *>(aux + size_t(m) * ld_aux + n);
+    }
+    TG_DEVICE void operator()(int m, int n, const float (&v)[4], u32x2 a, int) const {
         u32x2 packed;
         if (mode == EPI_RESIDUAL) {
             // y = RN(RN(acc) + residual): the bf16 add of cuda/mma.cuh:95-97
-            const u32x2 r = *reinterpret_cast<const u32x2 *>(aux + size_t(m) * ld_aux + n);
-            packed.x = pack_bf16(round_bf16(v[0]) + bf16_lo(r.x), round_bf16(v[1]) + bf16_hi(r.x));
-            packed.y = pack_bf16(round_bf16(v[2]) + bf16_lo(r.y), round_bf16(v[3]) + bf16_hi(r.y));
+            packed.x = pack_bf16(round_bf16(v[0]) + bf16_lo(a.x), round_bf16(v[1]) + bf16_hi(a.x));
+            packed.y = pack_bf16(round_bf16(v[2]) + bf16_lo(a.y), round_bf16(v[3]) + bf16_hi(a.y));
         } else if (mode == EPI_GELU_BWD) {
             // du = RN(RN(acc) * gelu'(u))
-            const u32x2 u = *reinterpret_cast<const u32x2 *>(aux + size_t(m) * ld_aux + n);
-            packed.x = pack_bf16(round_bf16(v[0]) * gelu_grad_f(bf16_lo(u.x)),
-                                 round_bf16(v[1]) * gelu_grad_f(bf16_hi(u.x)));
-            packed.y = pack_bf16(round_bf16(v[2]) * gelu_grad_f(bf16_lo(u.y)),
-                                 round_bf16(v[3]) * gelu_grad_f(bf16_hi(u.y)));
+            packed.x = pack_bf16(round_bf16(v[0]) * gelu_grad_f(bf16_lo(a.x)),
+                                 round_bf16(v[1]) * gelu_grad_f(bf16_hi(a.x)));
+            packed.y = pack_bf16(round_bf16(v[2]) * gelu_grad_f(bf16_lo(a.y)),
+                                 round_bf16(v[3]) * gelu_grad_f(bf16_hi(a.y)));
         } else {
             packed.x = pack_bf16(v[0], v[1]);
             packed.y = pack_bf16(v[2], v[3]);
@@ -65,11 +70,14 @@ struct EpilogueBf16 {
 };
 
 struct EpilogueF32 {
+    static constexpr bool AUX = false;
     float *out;
     int ld_out;
     size_t split_stride; // elements between split-K slabs
     int accumulate;      // only honoured when there is a single split
-    TG_DEVICE void operator()(int m, int n, const float (&v)[4], int split) const {
+    TG_DEVICE bool wants_aux() const { return false; }
+    TG_DEVICE u32x2 load_aux(int, int) const { return u32x2{0, 0}; }
+    TG_DEVICE void operator()(int m, int n, const float (&v)[4], u32x2, int split) const {
         f32x4 *p = reinterpret_cast<f32x4 *>(out + split * split_stride + size_t(m) * ld_out + n);
         f32x4 value = {v[0], v[1], v[2], v[3]};
         if (accumulate)
@@ -277,7 +285,20 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     acc[i][j][r] = 0.f;
+        const int out_m = m0 + wm + (lane & 31), out_n = n0 + wn + (lane >> 5) * 4;
+        u32x2 aux[Epilogue::AUX ? FM : 1][Epilogue::AUX ? FN : 1][4];
+        const int aux_at = nk > 2 ? nk - 2 : 0;
         for (int kt = 0; kt < nk; ++kt) {
+            if (Epilogue::AUX && kt == aux_at && epilogue.wants_aux()) {
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            aux[Epilogue::AUX ? i : 0][Epilogue::AUX ? j : 0][q] =
+                                epilogue.load_aux(out_m + i * 32, out_n + j * 32 + q * 8);
+            }
             // in flight now: the stage being consumed (landed), then inflight-1 younger ones; the next one
             // must land too
             wait_stages(inflight >= 2 ? inflight - 2 : 0);
@@ -300,7 +321,6 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[j], af1[i], acc[i][j], 0, 0, 0);
             c_slot = next_slot;
         }
-        const int out_m = m0 + wm + (lane & 31), out_n = n0 + wn + (lane >> 5) * 4;
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -309,7 +329,8 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
                 for (int q = 0; q < 4; ++q) {
                     const float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
                                         acc[i][j][q * 4 + 3]};
-                    epilogue(out_m + i * 32, out_n + j * 32 + q * 8, v, split);
+                    epilogue(out_m + i * 32, out_n + j * 32 + q * 8, v,
+                             aux[Epilogue::AUX ? i : 0][Epilogue::AUX ? j : 0][q], split);
                 }
     }
     wait_vmcnt<0>();
@@ -426,7 +447,7 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
         check_operand(X, ldx, "X");
         check_operand(W, ldw, "W");
         check_operand(Y, ldy, "Y");
-        EpilogueBf16 e{Y, ldy, nullptr, 0, nullptr, 0, EPI_PLAIN, 0};
+        EpilogueBf16 e{Y, ldy, nullptr, 0, nullptr, 0, EPI_PLAIN};
         if (residual) {
             check_operand(residual, ldr, "residual");
             e.aux = residual, e.ld_aux = ldr, e.mode = EPI_RESIDUAL;
@@ -449,7 +470,7 @@ extern "C" int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uin
         check_operand(dY, lddy, "dY");
         check_operand(W, ldw, "W");
         check_operand(dX, lddx, "dX");
-        EpilogueBf16 e{dX, lddx, nullptr, 0, nullptr, 0, EPI_PLAIN, 0};
+        EpilogueBf16 e{dX, lddx, nullptr, 0, nullptr, 0, EPI_PLAIN};
         if (gelu_pre) {
             check_operand(gelu_pre, ldu, "gelu_pre");
             e.aux = gelu_pre, e.ld_aux = ldu, e.mode = EPI_GELU_BWD;
