@@ -38,6 +38,13 @@ TGK_API int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint16_t
                  const uint16_t *W, int ldw, uint16_t *Y, int ldy, const uint16_t *residual, int ldr,
                  uint16_t *gelu_out, int ldg);
 
+/* The same forward projection with the weight given transposed, Wt[K][N] (leading dimension ldwt):
+ * the copy engine then moves whole rows of Wt instead of 64-byte pieces of W, which is markedly
+ * faster on the wide projections.  Same epilogues and shape rules as tgk_gemm_fwd. */
+TGK_API int tgk_gemm_fwd_t(hipStream_t stream, int M, int N, int K, const uint16_t *X, int ldx,
+                           const uint16_t *Wt, int ldwt, uint16_t *Y, int ldy, const uint16_t *residual,
+                           int ldr, uint16_t *gelu_out, int ldg);
+
 /* Input gradient, replaces matmul + cast_result as used by linear_backward
  * (cuda/ops.cuh:30-55, :115).
  *   dX[M][K] = RN_bf16( dY[M][N] . W[N][K] )
@@ -112,6 +119,13 @@ TGK_API size_t tgk_layernorm_bwd_workspace(int rows, int D);
  * write_grad != 0 overwrites the logits with RN_bf16((softmax - onehot) * inv_count). */
 TGK_API int tgk_cross_entropy(hipStream_t stream, int rows, int vocab, uint16_t *logits, const uint8_t *y,
                               float *loss, float *logits_f32, float inv_count, int write_grad);
+
+/* out[c][r] = in[r][c] for `count` row-major bf16 matrices that sit at the same element offset in
+ * `in` and `out` (the engine's transposed copy of the compute weights).  jobs: device array of
+ * {int64 offset; int32 rows, cols, first_tile, pad} with rows, cols multiples of 64 and
+ * first_tile the running count of 64x64 tiles; total_tiles = their sum. */
+TGK_API int tgk_transpose_batch(hipStream_t stream, const uint16_t *in, uint16_t *out, const void *jobs,
+                                int count, int total_tiles);
 
 /* partials[i] = sum of squares of block i's share of g (cuda/trainer.cuh:35-46); count <= 4096. */
 TGK_API int tgk_sumsq_partials(hipStream_t stream, const float *g, size_t n, float *partials, int count);

@@ -48,6 +48,46 @@ def test_forward_plain_residual_gelu(orc, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", SHAPES)
+def test_forward_with_transposed_weights(orc, M, N, K):
+    """tgk_gemm_fwd_t (Wt[K][N]) against the checker and against tgk_gemm_fwd; the batched transpose
+    that produces Wt is exact."""
+    lib = library()
+    rng = np.random.default_rng(M * 5 + N + K)
+    x, xh = to_bf16_device(rng.standard_normal((M, K)))
+    w, wh = to_bf16_device(rng.standard_normal((N, K)))
+    r, rh = to_bf16_device(rng.standard_normal((M, N)) * 4)
+    # two matrices in one buffer, transposed by one launch
+    other, oh = to_bf16_device(rng.standard_normal((64, 128)))
+    flat = torch.cat([w.flatten(), other.flatten()])
+    out = torch.zeros_like(flat)
+    jobs = np.zeros(2, dtype=[("offset", np.int64), ("rows", np.int32), ("cols", np.int32),
+                              ("first_tile", np.int32), ("pad", np.int32)])
+    jobs[0] = (0, N, K, 0, 0)
+    jobs[1] = (N * K, 64, 128, (N // 64) * (K // 64), 0)
+    jd = torch.from_numpy(jobs.view(np.uint8)).cuda()
+    check(lib.tgk_transpose_batch(stream(), flat.data_ptr(), out.data_ptr(), jd.data_ptr(), 2,
+                                  (N // 64) * (K // 64) + 2))
+    sync()
+    wt = out[:N * K].view(K, N)
+    assert torch.equal(wt, w.t().contiguous())
+    assert torch.equal(out[N * K:].view(128, 64), other.t().contiguous())
+    y = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    g = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    check(lib.tgk_gemm_fwd_t(stream(), M, N, K, x.data_ptr(), K, wt.data_ptr(), N, y.data_ptr(), N, None, 0, None, 0))
+    sync()
+    assert rel(host(y), orc.gemm_fwd(xh, wh)) < 1e-2
+    assert torch.equal(y, run_fwd(x, w)[0])  # same products, same summation order
+    check(lib.tgk_gemm_fwd_t(stream(), M, N, K, x.data_ptr(), K, wt.data_ptr(), N, y.data_ptr(), N, r.data_ptr(), N,
+                             None, 0))
+    sync()
+    assert rel(host(y), orc.gemm_fwd(xh, wh, residual=rh)) < 1e-2
+    check(lib.tgk_gemm_fwd_t(stream(), M, N, K, x.data_ptr(), K, wt.data_ptr(), N, y.data_ptr(), N, None, 0,
+                             g.data_ptr(), N))
+    sync()
+    assert rel(host(g), orc.gelu_fwd(orc.gemm_fwd(xh, wh))) < 1e-2
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
 def test_dgrad_and_fused_gelu_backward(orc, M, N, K):
     # dX[M][K] = dY[M][N] W[N][K]; here the tiled output dims are (M, K), the reduced one is N
     M, K, N = M, N, K

@@ -17,6 +17,8 @@ vp, i32, i64, f32, sz = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_size_t
 KERNEL_ABI = {
     "tgk_error": (C.c_char_p, []),
     "tgk_gemm_fwd": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
+    "tgk_gemm_fwd_t": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
+    "tgk_transpose_batch": (i32, [vp, vp, vp, vp, i32, i32]),
     "tgk_gemm_dgrad": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
     "tgk_gemm_wgrad": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, i32, vp, sz]),
     "tgk_gemm_wgrad_workspace": (sz, [i32, i32, i32]),

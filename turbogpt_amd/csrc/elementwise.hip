@@ -452,6 +452,49 @@ __global__ __launch_bounds__(256) void position_means_kernel(const float *__rest
     out[p] = float(sum / batch);
 }
 
+// ---- batched bf16 transposes ------------------------------------------------------------------
+// out[c][r] = in[r][c] for a list of row-major matrices that live at the same offset in `in` and
+// `out`.  64x64 tiles through LDS; a block finds its matrix from the running tile counts.
+struct TransposeJob {
+    int64_t offset; // element offset of the matrix in both buffers
+    int rows, cols; // of the source
+    int first_tile; // running count of 64x64 tiles before this matrix
+    int pad;
+};
+__global__ __launch_bounds__(256) void transpose_batch_kernel(const bf16_t *__restrict__ in,
+                                                              bf16_t *__restrict__ out,
+                                                              const TransposeJob *__restrict__ jobs, int count) {
+    __shared__ bf16_t tile[64][66];
+    int lo = 0, hi = count - 1; // last job whose first_tile <= blockIdx.x
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (jobs[mid].first_tile <= int(blockIdx.x))
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    const TransposeJob job = jobs[lo];
+    const int t = blockIdx.x - job.first_tile, tiles_c = job.cols >> 6;
+    const int r0 = (t / tiles_c) << 6, c0 = (t % tiles_c) << 6;
+    const bf16_t *src = in + job.offset;
+    bf16_t *dst = out + job.offset;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 column pairs x 8 rows
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = ty + i * 8;
+        const uint32_t pair = *reinterpret_cast<const uint32_t *>(src + size_t(r0 + r) * job.cols + c0 + tx * 2);
+        tile[r][tx * 2] = bf16_t(pair);
+        tile[r][tx * 2 + 1] = bf16_t(pair >> 16);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int c = ty + i * 8; // source column = destination row
+        const uint32_t pair = uint32_t(tile[tx * 2][c]) | (uint32_t(tile[tx * 2 + 1][c]) << 16);
+        *reinterpret_cast<uint32_t *>(dst + size_t(c0 + c) * job.rows + r0 + tx * 2) = pair;
+    }
+}
+
 int grid_for(size_t work_items, int per_block, int cap = 4096) {
     const size_t blocks = (work_items + per_block - 1) / per_block;
     return int(blocks < size_t(cap) ? (blocks ? blocks : 1) : cap);
@@ -638,5 +681,15 @@ extern "C" int tgk_position_means(hipStream_t stream, const float *token_loss, i
         hipLaunchKernelGGL(position_means_kernel, dim3((context + 255) / 256), dim3(256), 0, stream, token_loss,
                            batch, context, out);
         check_hip(hipGetLastError(), "position_means launch: ");
+    });
+}
+
+extern "C" int tgk_transpose_batch(hipStream_t stream, const uint16_t *in, uint16_t *out, const void *jobs,
+                                   int count, int total_tiles) {
+    return guarded([&] {
+        require(in && out && jobs && count > 0 && total_tiles > 0, "transpose_batch: missing operand");
+        hipLaunchKernelGGL(transpose_batch_kernel, dim3(total_tiles), dim3(256), 0, stream, in, out,
+                           static_cast<const TransposeJob *>(jobs), count);
+        check_hip(hipGetLastError(), "transpose_batch launch: ");
     });
 }

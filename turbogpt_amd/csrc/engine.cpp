@@ -66,6 +66,9 @@ struct Engine {
     int compute_units = 0;
 
     uint16_t *weight_hi = nullptr, *weight_lo = nullptr;
+    uint16_t *weight_t = nullptr; // every matrix of weight_hi transposed ([In][Out]), same offsets
+    void *transpose_jobs = nullptr;
+    int transpose_count = 0, transpose_tiles = 0;
     float *momentum = nullptr, *variance = nullptr, *gradient = nullptr;
     float *norm_partials = nullptr, *token_losses = nullptr, *loss_history = nullptr;
     int64_t *segment_starts = nullptr;
@@ -156,6 +159,11 @@ struct Engine {
 
     const uint16_t *w(int64_t offset) const { return weight_hi + offset; }
     const uint16_t *wl(int64_t offset) const { return weight_lo + offset; }
+    const uint16_t *wt(int64_t offset) const { return weight_t + offset; }
+    // forward projections read the transposed weights: call after every change of weight_hi
+    void refresh_transposed() {
+        ok(tgk_transpose_batch(stream, weight_hi, weight_t, transpose_jobs, transpose_count, transpose_tiles));
+    }
 
     // cuda/model.cuh:8-59.  evaluate: logits stay logits; otherwise they are replaced by dlogits.
     void forward(const uint8_t *tokens_in, const uint8_t *targets, bool with_gradient, float *logits_out) {
@@ -168,18 +176,18 @@ struct Engine {
             LayerBuffers &b = layers[l];
             OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, x[l], w(p.ln1_g), wl(p.ln1_g), w(p.ln1_b), wl(p.ln1_b), b.n1,
                                  config.ln_eps));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, 3 * d, d, b.n1, d, w(p.qkv), d, b.qkv, 3 * d, nullptr, 0, nullptr, 0));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, 3 * d, d, b.n1, d, wt(p.qkv), 3 * d, b.qkv, 3 * d, nullptr, 0, nullptr, 0));
             OP(TG_CLASS_ATTN_FWD, tgk_attn_fwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
                             3 * d, b.o, d, b.lse, scale));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, d, b.o, d, w(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, d, d, b.o, d, wt(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
             OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, b.mid, w(p.ln2_g), wl(p.ln2_g), w(p.ln2_b), wl(p.ln2_b), b.n2,
                                  config.ln_eps));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, F, d, b.n2, d, w(p.mlp_up), d, b.u, F, nullptr, 0, b.a, F));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, F, b.a, F, w(p.mlp_down), F, x[l + 1], d, b.mid, d, nullptr, 0));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, F, d, b.n2, d, wt(p.mlp_up), F, b.u, F, nullptr, 0, b.a, F));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, d, F, b.a, F, wt(p.mlp_down), d, x[l + 1], d, b.mid, d, nullptr, 0));
         }
         OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, x[c.depth], w(layout.lnf_g), wl(layout.lnf_g), w(layout.lnf_b),
                              wl(layout.lnf_b), nf, config.ln_eps));
-        OP(TG_CLASS_HEAD, tgk_gemm_fwd(stream, M, V, d, nf, d, w(layout.head), d, logits, V, nullptr, 0, nullptr, 0));
+        OP(TG_CLASS_HEAD, tgk_gemm_fwd_t(stream, M, V, d, nf, d, wt(layout.head), V, logits, V, nullptr, 0, nullptr, 0));
         OP(TG_CLASS_OTHER, tgk_cross_entropy(stream, M, V, logits, targets, token_losses, logits_out, 1.0f / float(M),
                              with_gradient ? 1 : 0));
     }
@@ -231,6 +239,8 @@ struct Engine {
         OP(TG_CLASS_OPTIMIZER, tgk_adamw(stream, size_t(layout.count), weight_hi, weight_lo, momentum, variance, gradient,
                      norm_partials, NormPartials, segment_starts, segment_flags, segments, lr, beta1, c.beta2,
                      c.epsilon, c.weight_decay, c.clip, at));
+        OP(TG_CLASS_OPTIMIZER, tgk_transpose_batch(stream, weight_hi, weight_t, transpose_jobs, transpose_count,
+                                                   transpose_tiles));
     }
     // one full training step; shared by tg_train and tg_profile_step
     void train_step(uint64_t at, float *history_row) {
@@ -278,6 +288,36 @@ void validate(const TgModelConfig &m) {
         throw std::runtime_error("inflight must be 1: the stale-gradient pipeline is not built");
     if (!(m.ln_eps > 0))
         throw std::runtime_error("ln_eps must be positive");
+}
+
+void build_transpose_jobs(Engine *e) {
+    struct Job {
+        int64_t offset;
+        int rows, cols, first_tile, pad;
+    };
+    std::vector<Job> jobs;
+    int tiles = 0;
+    const auto add = [&](int64_t offset, int rows, int cols) {
+        jobs.push_back({offset, rows, cols, tiles, 0});
+        tiles += (rows / 64) * (cols / 64);
+    };
+    const TgParameterLayout &p = e->layout;
+    const int d = e->config.d_model, F = e->config.ffn, V = e->config.vocab;
+    for (int l = 0; l < e->config.base.depth; ++l) {
+        const TgLayerParameters &b = p.layers[l];
+        add(b.qkv, 3 * d, d);
+        add(b.attn_out, d, d);
+        add(b.mlp_up, F, d);
+        add(b.mlp_down, d, F);
+    }
+    add(p.head, V, d);
+    Job *device = nullptr;
+    e->allocate(device, jobs.size(), false);
+    e->upload(device, jobs.data(), jobs.size());
+    e->sync();
+    e->transpose_jobs = device;
+    e->transpose_count = int(jobs.size());
+    e->transpose_tiles = tiles;
 }
 
 void build_segments(Engine *e) {
@@ -346,6 +386,7 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
         const size_t F = size_t(model->ffn), V = size_t(model->vocab);
         e->allocate(e->weight_hi, P);
         e->allocate(e->weight_lo, P);
+        e->allocate(e->weight_t, P);
         e->allocate(e->momentum, P);
         e->allocate(e->variance, P);
         e->allocate(e->gradient, P);
@@ -355,6 +396,7 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
         e->allocate(e->input, M);
         e->allocate(e->target, M);
         build_segments(e);
+        build_transpose_jobs(e);
         e->x.resize(c.depth + 1);
         e->layers.resize(c.depth);
         for (int l = 0; l <= c.depth; ++l)
@@ -441,6 +483,7 @@ TG_API int tg_set_weights(Engine *e, const float *weights) {
         e->upload(e->weight_lo, low.data(), n);
         check_hip(hipMemsetAsync(e->momentum, 0, n * 4, e->stream));
         check_hip(hipMemsetAsync(e->variance, 0, n * 4, e->stream));
+        e->refresh_transposed();
         e->step = 0;
         e->sync();
     });

@@ -459,6 +459,31 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
     });
 }
 
+extern "C" int tgk_gemm_fwd_t(hipStream_t stream, int M, int N, int K, const uint16_t *X, int ldx,
+                              const uint16_t *Wt, int ldwt, uint16_t *Y, int ldy, const uint16_t *residual,
+                              int ldr, uint16_t *gelu_out, int ldg) {
+    return guarded([&] {
+        require(M > 0 && N > 0 && K > 0, "gemm_fwd_t: empty shape");
+        require(K % BK == 0, "gemm_fwd_t: K must be a multiple of 32");
+        const Tile tile = choose_tile(M, N);
+        require(tile != TILE_NONE, "gemm_fwd_t: M must be a multiple of 128 and N of 128 or 192");
+        require(!(residual && gelu_out), "gemm_fwd_t: residual and GELU epilogues are exclusive");
+        check_operand(X, ldx, "X");
+        check_operand(Wt, ldwt, "Wt");
+        check_operand(Y, ldy, "Y");
+        EpilogueBf16 e{Y, ldy, nullptr, 0, nullptr, 0, EPI_PLAIN};
+        if (residual) {
+            check_operand(residual, ldr, "residual");
+            e.aux = residual, e.ld_aux = ldr, e.mode = EPI_RESIDUAL;
+        } else if (gelu_out) {
+            check_operand(gelu_out, ldg, "gelu_out");
+            e.out2 = gelu_out, e.ld_out2 = ldg, e.mode = EPI_GELU;
+        }
+        // B(n, k) = Wt[k][n]: k-strided, whole 384-byte rows per copy instead of 64-byte pieces
+        dispatch_gemm<true, false>(stream, tile, X, ldx, Wt, ldwt, M, N, K, 1, e);
+    });
+}
+
 extern "C" int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uint16_t *dY, int lddy,
                               const uint16_t *W, int ldw, uint16_t *dX, int lddx,
                               const uint16_t *gelu_pre, int ldu) {
