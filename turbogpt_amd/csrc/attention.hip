@@ -85,20 +85,138 @@ TG_DEVICE void tile_store(const u32x4 (&regs)[2], bf16_t *tile, int tid) {
     }
 }
 
+// ---- swizzled 64 x 64 LDS tiles filled by wave-wide global -> LDS copies -------------------------
+// 128-byte rows, no padding (a copy fills 1 KiB contiguously); the 16-byte chunk c of row r sits at
+// chunk c ^ swz(r).  swz is chosen so that both access patterns are bank-conflict free: fragments along
+// the rows (16 consecutive rows, one chunk each) and transposing reads along the columns (4 consecutive
+// rows, 32 bytes each).
+constexpr int TILE_ELEMS = 64 * 64;
+TG_DEVICE int swz(int row) {
+    return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+}
+// this wave's two copies (regions wave and wave+4, 8 rows each) of a 64-row tile starting at `base`
+TG_DEVICE void tile_copy_async(uint32_t lds_tile, const bf16_t *base, int ld, int wave, int lane) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int region = wave + 4 * j, row = region * 8 + (lane >> 3), chunk = (lane & 7) ^ swz(row);
+        async_copy16(__builtin_amdgcn_readfirstlane(lds_tile + region * 1024), base + size_t(row) * ld + chunk * 8);
+    }
+}
+// rows row0 + lane%32, k = k0 + 8*(lane/32) .. +7   (k0 a multiple of 16)
+TG_DEVICE bf16x8 sfrag_rows(const bf16_t *tile, int row0, int k0, int lane) {
+    const int row = row0 + (lane & 31), chunk = ((k0 >> 3) + (lane >> 5)) ^ swz(row);
+    return *reinterpret_cast<const bf16x8 *>(tile + row * 64 + chunk * 8);
+}
+// column col0 + lane%32, rows krow0 + 4g + {0..3} and krow0 + 8 + 4g + {0..3} (the acc_row order)
+TG_DEVICE bf16x8 sfrag_cols(const bf16_t *tile, int krow0, int col0, int lane) {
+    const int g = lane >> 5, blk = (lane >> 4) & 1, i = lane & 15;
+    const int r = krow0 + 4 * g + (i >> 2), col = col0 + 16 * blk + 4 * (i & 3);
+    const bf16_t *p0 = tile + r * 64 + (((col >> 3) ^ swz(r)) << 3) + (col & 7);
+    const bf16_t *p1 = tile + (r + 8) * 64 + (((col >> 3) ^ swz(r + 8)) << 3) + (col & 7);
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p0));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p1));
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, both);
+}
+
+// The swizzle terms of both fragment kinds depend on the lane only (swz(row + 32) = swz(row);
+// swz(r + 16) = swz(r)), so a kernel computes these element offsets once and adds compile-time
+// constants per k-step / tile inside its loops.
+struct RowFragOffsets { // sfrag_rows(tile, mt * 32, ks * 16, lane) = tile + at[ks] + mt * 32 * 64
+    int at[4];
+    TG_DEVICE explicit RowFragOffsets(int lane) {
+        const int row = lane & 31;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+            at[ks] = row * 64 + (((ks * 2 + (lane >> 5)) ^ swz(row)) << 3);
+    }
+    TG_DEVICE bf16x8 load(const bf16_t *tile, int mt, int ks) const {
+        return *reinterpret_cast<const bf16x8 *>(tile + at[ks] + mt * 32 * 64);
+    }
+};
+struct ColFragOffsets { // sfrag_cols(tile, kk * 16, dt * 32, lane): rows +kk*16 are a constant offset
+    int lo[2], hi[2];
+    TG_DEVICE explicit ColFragOffsets(int lane) {
+        const int g = lane >> 5, blk = (lane >> 4) & 1, i = lane & 15;
+        const int r = 4 * g + (i >> 2);
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+            const int col = dt * 32 + 16 * blk + 4 * (i & 3);
+            lo[dt] = r * 64 + (((col >> 3) ^ swz(r)) << 3) + (col & 7);
+            hi[dt] = (r + 8) * 64 + (((col >> 3) ^ swz(r + 8)) << 3) + (col & 7);
+        }
+    }
+    TG_DEVICE bf16x8 load(const bf16_t *tile, int kk, int dt) const {
+        const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(tile + lo[dt] + kk * 16 * 64));
+        const s16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(tile + hi[dt] + kk * 16 * 64));
+        const s16x8 both = __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, both);
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
-// forward: block = 128 queries (4 waves x 32), key/value tiles of 64, heavy (late) tiles first
+// forward: block = 128 queries (4 waves x 32), key/value tiles of 64 in three LDS stages filled by
+// asynchronous copies issued two tiles ahead; heavy (late) query tiles first.  The tile loop is
+// unrolled by the stage count so every LDS address is a per-lane constant plus an immediate; three
+// resident waves per SIMD overlap one wave's softmax with another's matrix work.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const bf16_t *__restrict__ Q,
+// Block placement.  The work of a causal tile grows with its index and consecutive block ids go to the
+// eight XCDs in turn, so a (tile, head, batch) grid whose tile extent is a multiple of 8 hands one XCD
+// all the heaviest tiles.  Instead each XCD takes every eighth (batch, head) pair with all of that
+// pair's tiles - which also keeps a pair's keys and values in one L2 - heaviest rank first.
+struct CausalBlock {
+    int rank, h, b;
+    bool live;
+};
+TG_DEVICE CausalBlock causal_block(int H, int pairs) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, per_xcd = (pairs + 7) >> 3;
+    const int pair = (slot % per_xcd) * 8 + xcd;
+    return {slot / per_xcd, pair % H, pair / H, pair < pairs};
+}
+unsigned causal_grid(int tiles, int pairs) {
+    return unsigned(tiles) * unsigned((pairs + 7) / 8) * 8u;
+}
+
+template <int N> struct Const {
+    static constexpr int value = N;
+};
+// Lanes i and i+32 own the two halves of one query's keys.  v_permlane32_swap of a value with itself
+// leaves the lower lanes' values in every lane of the first result and the upper lanes' in the second.
+TG_DEVICE float halves_max(float x) {
+    const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
+}
+TG_DEVICE float halves_sum(float x) {
+    const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(both[0]) + __uint_as_float(both[1]);
+}
+
+__global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restrict__ Q,
                                                           const bf16_t *__restrict__ K,
                                                           const bf16_t *__restrict__ V, int ld,
                                                           bf16_t *__restrict__ O, int ldo,
                                                           float *__restrict__ LSE, int T, int H,
-                                                          float c) {
-    __shared__ __align__(16) bf16_t sK[2][64 * LS], sV[2][64 * LS];
-    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128, h = blockIdx.y, b = blockIdx.z;
+                                                          int pairs, float c) {
+    __shared__ __align__(1024) bf16_t stages[3][2][TILE_ELEMS]; // [stage][K | V]
+    const CausalBlock block = causal_block(H, pairs);
+    if (!block.live)
+        return;
+    const int q0 = (T / 128 - 1 - block.rank) * 128, h = block.h, b = block.b;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5;
     const int wave_q0 = q0 + wave * 32, qrow = wave_q0 + (lane & 31);
     const size_t token0 = size_t(b) * T;
+    const int tiles = (q0 + 128) / 64;
+    const int my_tiles = wave_q0 / 64 + 1; // tiles with a key visible to this wave (wave uniform)
+    const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
+    const uint32_t lds0 = lds_address(&stages[0][0][0]);
+    auto produce = [&](int stage, int j) {
+        const uint32_t slot = lds0 + uint32_t(stage) * (2 * TILE_ELEMS * 2);
+        tile_copy_async(slot, kbase + size_t(j) * 64 * ld, ld, wave, lane);
+        tile_copy_async(slot + TILE_ELEMS * 2, vbase + size_t(j) * 64 * ld, ld, wave, lane);
+    };
+    produce(0, 0);
+    if (tiles > 1)
+        produce(1, 1);
 
     bf16x8 qf[4];
     {
@@ -108,78 +226,80 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const bf16_t *__restri
             qf[ks] = *reinterpret_cast<const bf16x8 *>(qp + ks * 16);
     }
     f32x16 o[2] = {zero16(), zero16()};
-    float m = -INFINITY, l = 0.f;
+    float m = -INFINITY, l = 0.f; // l: this lane's half of the keys only, halves are joined at the end
+    const RowFragOffsets krows(lane);
+    const ColFragOffsets vcols(lane);
 
-    const int tiles = (q0 + 128) / 64;
-    const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
-    u32x4 kr[2], vr[2];
-    tile_load(kr, kbase, ld, tid);
-    tile_load(vr, vbase, ld, tid);
-    tile_store(kr, sK[0], tid);
-    tile_store(vr, sV[0], tid);
-    __syncthreads();
-    for (int j = 0; j < tiles; ++j) {
-        const int cur = j & 1, kv0 = j * 64;
-        const bool more = j + 1 < tiles;
-        if (more) {
-            tile_load(kr, kbase + size_t(kv0 + 64) * ld, ld, tid);
-            tile_load(vr, vbase + size_t(kv0 + 64) * ld, ld, tid);
-        }
-        if (kv0 <= wave_q0 + 31) { // some key of this tile is visible to this wave (wave uniform)
-            f32x16 s[2] = {zero16(), zero16()};
+    auto step = [&](auto stage_tag, int j) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        // tile j was issued two steps ago; only tile j+1's four copies may still be in flight
+        if (j + 1 < tiles)
+            wait_vmcnt<4>();
+        else
+            wait_vmcnt<0>();
+        __syncthreads(); // tile j visible to every wave; everyone is done with tile j-1's stage
+        if (j + 2 < tiles)
+            produce((STAGE + 2) % 3, j + 2);
+        if (j >= my_tiles)
+            return;
+        const bf16_t *kt = stages[STAGE][0], *vt = stages[STAGE][1];
+        const int kv0 = j * 64;
+        f32x16 s[2] = {zero16(), zero16()};
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
-                    s[mt] = mfma(frag_rows(sK[cur], mt * 32, ks * 16, lane), qf[ks], s[mt]);
-            if (kv0 + 63 > wave_q0) { // diagonal tile: hide keys after the query
-#pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (kv0 + mt * 32 + acc_row(r, g) > qrow)
-                            s[mt][r] = -INFINITY;
-            }
-            float mx = -INFINITY;
+            for (int mt = 0; mt < 2; ++mt)
+                s[mt] = mfma(krows.load(kt, mt, ks), qf[ks], s[mt]);
+        if (kv0 + 63 > wave_q0) { // diagonal tile: hide keys after the query
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    mx = fmaxf(mx, s[mt][r]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m, mx * c);
-            const float alpha = exp2_fast(m - m_new);
-            float sum = 0.f;
+                    if (kv0 + mt * 32 + acc_row(r, g) > qrow)
+                        s[mt][r] = -INFINITY;
+        }
+        float mx = -INFINITY;
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
+        for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float p = exp2_fast(fmaf(s[mt][r], c, -m_new));
-                    s[mt][r] = p;
-                    sum += p;
-                }
-            sum += __shfl_xor(sum, 32, 64);
-            l = l * alpha + sum;
-            m = m_new;
+            for (int r = 0; r < 16; ++r)
+                mx = fmaxf(mx, s[mt][r]);
+        mx = halves_max(mx);
+        const float m_new = fmaxf(m, mx * c);
+        const float alpha = exp2_fast(m - m_new);
+        float sum = 0.f;
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = exp2_fast(fmaf(s[mt][r], c, -m_new));
+                s[mt][r] = p;
+                sum += p;
+            }
+        l = l * alpha + sum;
+        if (__builtin_amdgcn_ballot_w64(m_new != m)) { // rescale only when some row's maximum moved
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     o[dt][r] *= alpha;
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                const bf16x8 pf = acc_to_frag(s[kk >> 1], kk & 1);
-#pragma unroll
-                for (int dt = 0; dt < 2; ++dt)
-                    o[dt] = mfma(frag_cols(sV[cur], kk * 16, dt * 32, lane), pf, o[dt]);
-            }
         }
-        if (more) {
-            tile_store(kr, sK[cur ^ 1], tid);
-            tile_store(vr, sV[cur ^ 1], tid);
+        m = m_new;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            const bf16x8 pf = acc_to_frag(s[kk >> 1], kk & 1);
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+                o[dt] = mfma(vcols.load(vt, kk, dt), pf, o[dt]);
         }
-        __syncthreads();
+    };
+    for (int j = 0; j < tiles; j += 3) { // tiles is even and block uniform
+        step(Const<0>{}, j);
+        step(Const<1>{}, j + 1);
+        if (j + 2 < tiles)
+            step(Const<2>{}, j + 2);
     }
+    l = halves_sum(l);
     const float inv = 1.0f / l;
     bf16_t *op = O + (token0 + qrow) * ldo + h * HD + 4 * g;
 #pragma unroll
@@ -228,9 +348,12 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
     const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
     const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ LSE,
     const float *__restrict__ delta, bf16_t *__restrict__ dK, bf16_t *__restrict__ dV, int lddq, int T,
-    int H, float scale) {
+    int H, int pairs, float scale) {
     __shared__ __align__(16) bf16_t sQ[2][64 * LS], sdO[2][64 * LS];
-    const int k0 = blockIdx.x * 128, h = blockIdx.y, b = blockIdx.z;
+    const CausalBlock block = causal_block(H, pairs);
+    if (!block.live)
+        return;
+    const int k0 = block.rank * 128, h = block.h, b = block.b; // early keys see the most queries
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5;
     const int wave_k0 = k0 + wave * 32, krow = wave_k0 + (lane & 31);
     const size_t token0 = size_t(b) * T;
@@ -332,9 +455,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
     const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ LSE,
-    const float *__restrict__ delta, bf16_t *__restrict__ dQ, int lddq, int T, int H, float scale) {
+    const float *__restrict__ delta, bf16_t *__restrict__ dQ, int lddq, int T, int H, int pairs,
+    float scale) {
     __shared__ __align__(16) bf16_t sK[2][64 * LS], sV[2][64 * LS];
-    const int q0 = (gridDim.x - 1 - blockIdx.x) * 128, h = blockIdx.y, b = blockIdx.z;
+    const CausalBlock block = causal_block(H, pairs);
+    if (!block.live)
+        return;
+    const int q0 = (T / 128 - 1 - block.rank) * 128, h = block.h, b = block.b;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5;
     const int wave_q0 = q0 + wave * 32, qrow = wave_q0 + (lane & 31);
     const size_t token0 = size_t(b) * T;
@@ -438,8 +565,8 @@ extern "C" int tgk_attn_fwd(hipStream_t stream, int B, int H, int T, int hd, con
         check_matrix(V, ld, "V");
         check_matrix(O, ldo, "O");
         require(lse && !(reinterpret_cast<uintptr_t>(lse) & 15), "attention: lse must be 16-byte aligned");
-        hipLaunchKernelGGL(attn_fwd_kernel, dim3(T / 128, H, B), dim3(256), 0, stream, Q, K, V, ld, O, ldo,
-                           lse, T, H, scale * LOG2E);
+        hipLaunchKernelGGL(attn_fwd_kernel, dim3(causal_grid(T / 128, B * H)), dim3(256), 0, stream, Q, K, V,
+                           ld, O, ldo, lse, T, H, B * H, scale * LOG2E);
         check_hip(hipGetLastError(), "attention forward launch: ");
     });
 }
@@ -471,10 +598,11 @@ extern "C" int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, con
         const int rows = B * T;
         hipLaunchKernelGGL(attn_delta_kernel, dim3((rows * H + 31) / 32), dim3(256), 0, stream, dO, lddo, O,
                            ldo, delta, T, H, rows);
-        hipLaunchKernelGGL(attn_bwd_dkdv_kernel, dim3(T / 128, H, B), dim3(256), 0, stream, Q, K, V, ld, dO,
-                           lddo, lse, delta, dK, dV, lddq, T, H, scale);
-        hipLaunchKernelGGL(attn_bwd_dq_kernel, dim3(T / 128, H, B), dim3(256), 0, stream, Q, K, V, ld, dO,
-                           lddo, lse, delta, dQ, lddq, T, H, scale);
+        const dim3 grid(causal_grid(T / 128, B * H));
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse, delta,
+                           dK, dV, lddq, T, H, B * H, scale);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse, delta,
+                           dQ, lddq, T, H, B * H, scale);
         check_hip(hipGetLastError(), "attention backward launch: ");
     });
 }

@@ -75,6 +75,20 @@ TG_DEVICE float wave_max(float x) {
     return x;
 }
 
+// One wave-wide global -> LDS copy of 16 bytes per lane (global_load_lds_dwordx4): lane l lands at
+// LDS byte address lds_base + 16*l, lds_base wave-uniform.  The compiler does not track these copies;
+// completion is awaited explicitly with wait_vmcnt<N>() ("at most N of this wave's vector-memory
+// operations still outstanding") before the barrier that publishes the data to the other waves.
+TG_DEVICE void async_copy16(uint32_t lds_base, const void *global) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(global) : "memory");
+}
+template <int N> TG_DEVICE void wait_vmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+TG_DEVICE uint32_t lds_address(const void *shared_pointer) {
+    return uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void *)shared_pointer));
+}
+
 // ---- host side ---------------------------------------------------------------------------
 extern thread_local std::string tg_last_error;
 

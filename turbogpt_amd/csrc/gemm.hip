@@ -91,14 +91,6 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-// one wave-wide 16-byte-per-lane global -> LDS copy: lane l lands at lds_base + 16*l
-TG_DEVICE void async_copy16(uint32_t lds_base, const void *global) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(global) : "memory");
-}
-template <int N> TG_DEVICE void wait_vmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
 // ---- k-contiguous operand tile: ROWS rows x 32 k, 64-byte rows, 16-byte chunk c of row r stored
 // at chunk c ^ ((r >> 2) & 3) ------------------------------------------------------------------
 template <int ROWS> struct TileKC {
@@ -176,7 +168,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
     constexpr int LA = TA::LOADS, LB = TB::LOADS, LOADS = LA + LB;
     constexpr int STAGE = TA::BYTES + TB::BYTES;
     extern __shared__ __align__(16) unsigned char smem[];
-    const uint32_t smem_base = uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) unsigned char *)smem));
+    const uint32_t smem_base = lds_address(smem);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
