@@ -82,7 +82,7 @@ def test_kernel_entry_points_validate_arguments_on_the_host():
     assert lib.tgk_gemm_fwd(None, 100, 128, 64, None, 64, None, 64, None, 128, None, 0, None, 0) == -1
     assert lib.tgk_attn_fwd(None, 1, 1, 100, 64, None, None, None, 192, None, 64, None, 0.125) == -1
     assert lib.tgk_gemm_wgrad_workspace(64, 100, 128) == 0
-    assert lib.tgk_attn_bwd_workspace(2, 3, 128) == 2 * 3 * 128 * 4
+    assert lib.tgk_attn_bwd_workspace(2, 3, 128) == 2 * (2 * 3 * 128 * 4)
     assert lib.tgk_layernorm_bwd_workspace(16384, 768) == 1024 * 2 * 768 * 4
 
 

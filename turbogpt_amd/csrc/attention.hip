@@ -20,7 +20,6 @@
 namespace {
 
 constexpr int HD = 64;      // head dimension
-constexpr int LS = HD + 8;  // LDS row stride in elements
 constexpr float LOG2E = 1.4426950408889634f, LN2 = 0.6931471805599453f;
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -41,22 +40,6 @@ TG_DEVICE f32x16 mfma(bf16x8 rows_to_regs, bf16x8 rows_to_lanes, f32x16 acc) {
 TG_DEVICE int acc_row(int r, int g) {
     return 8 * (r >> 2) + 4 * g + (r & 3);
 }
-// 16-byte fragment of a [row][k] LDS tile: row = row0 + lane%32, k = k0 + 8*(lane/32) .. +7
-TG_DEVICE bf16x8 frag_rows(const bf16_t *tile, int row0, int k0, int lane) {
-    return *reinterpret_cast<const bf16x8 *>(tile + (row0 + (lane & 31)) * LS + k0 + (lane >> 5) * 8);
-}
-// Fragment of the same tile read along its rows: the lane gets column col0 + lane%32 and the 8
-// rows  krow0 + 4g + {0..3}  and  krow0 + 8 + 4g + {0..3}  - exactly the rows that accumulator
-// registers 8*kk2 .. 8*kk2+7 of a 32x32 tile hold (acc_row), so a converted accumulator and this
-// fragment agree on the order of the reduced index.
-TG_DEVICE bf16x8 frag_cols(const bf16_t *tile, int krow0, int col0, int lane) {
-    const int g = lane >> 5, blk = (lane >> 4) & 1, i = lane & 15;
-    const bf16_t *p = tile + (krow0 + 4 * g + (i >> 2)) * LS + col0 + 16 * blk + 4 * (i & 3);
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 8 * LS));
-    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, both);
-}
 // registers 8*kk2 .. 8*kk2+7 of an fp32 accumulator as a bf16 operand fragment
 TG_DEVICE bf16x8 acc_to_frag(const f32x16 &acc, int kk2) {
     bf16x8 f;
@@ -67,22 +50,6 @@ TG_DEVICE bf16x8 acc_to_frag(const f32x16 &acc, int kk2) {
 }
 TG_DEVICE float exp2_fast(float x) {
     return __builtin_amdgcn_exp2f(x);
-}
-
-// 64 rows x 64 columns of a [token][ld] bf16 matrix -> registers -> LDS tile, 256 threads
-TG_DEVICE void tile_load(u32x4 (&regs)[2], const bf16_t *base, int ld, int tid) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int c = tid + i * 256, row = c >> 3, kc = c & 7;
-        regs[i] = *reinterpret_cast<const u32x4 *>(base + size_t(row) * ld + kc * 8);
-    }
-}
-TG_DEVICE void tile_store(const u32x4 (&regs)[2], bf16_t *tile, int tid) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int c = tid + i * 256, row = c >> 3, kc = c & 7;
-        *reinterpret_cast<u32x4 *>(tile + row * LS + kc * 8) = regs[i];
-    }
 }
 
 // ---- swizzled 64 x 64 LDS tiles filled by wave-wide global -> LDS copies -------------------------
@@ -102,27 +69,11 @@ TG_DEVICE void tile_copy_async(uint32_t lds_tile, const bf16_t *base, int ld, in
         async_copy16(__builtin_amdgcn_readfirstlane(lds_tile + region * 1024), base + size_t(row) * ld + chunk * 8);
     }
 }
-// rows row0 + lane%32, k = k0 + 8*(lane/32) .. +7   (k0 a multiple of 16)
-TG_DEVICE bf16x8 sfrag_rows(const bf16_t *tile, int row0, int k0, int lane) {
-    const int row = row0 + (lane & 31), chunk = ((k0 >> 3) + (lane >> 5)) ^ swz(row);
-    return *reinterpret_cast<const bf16x8 *>(tile + row * 64 + chunk * 8);
-}
-// column col0 + lane%32, rows krow0 + 4g + {0..3} and krow0 + 8 + 4g + {0..3} (the acc_row order)
-TG_DEVICE bf16x8 sfrag_cols(const bf16_t *tile, int krow0, int col0, int lane) {
-    const int g = lane >> 5, blk = (lane >> 4) & 1, i = lane & 15;
-    const int r = krow0 + 4 * g + (i >> 2), col = col0 + 16 * blk + 4 * (i & 3);
-    const bf16_t *p0 = tile + r * 64 + (((col >> 3) ^ swz(r)) << 3) + (col & 7);
-    const bf16_t *p1 = tile + (r + 8) * 64 + (((col >> 3) ^ swz(r + 8)) << 3) + (col & 7);
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p0));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p1));
-    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, both);
-}
-
 // The swizzle terms of both fragment kinds depend on the lane only (swz(row + 32) = swz(row);
 // swz(r + 16) = swz(r)), so a kernel computes these element offsets once and adds compile-time
 // constants per k-step / tile inside its loops.
-struct RowFragOffsets { // sfrag_rows(tile, mt * 32, ks * 16, lane) = tile + at[ks] + mt * 32 * 64
+// operand fragment along the rows: row mt*32 + lane%32, k = ks*16 + 8*(lane/32) .. +7
+struct RowFragOffsets {
     int at[4];
     TG_DEVICE explicit RowFragOffsets(int lane) {
         const int row = lane & 31;
@@ -134,7 +85,10 @@ struct RowFragOffsets { // sfrag_rows(tile, mt * 32, ks * 16, lane) = tile + at[
         return *reinterpret_cast<const bf16x8 *>(tile + at[ks] + mt * 32 * 64);
     }
 };
-struct ColFragOffsets { // sfrag_cols(tile, kk * 16, dt * 32, lane): rows +kk*16 are a constant offset
+// operand fragment along the columns (transposing reads): column dt*32 + lane%32 and the 8 rows
+// kk*16 + 4g + {0..3}, kk*16 + 8 + 4g + {0..3} - the rows that accumulator registers 8*(kk%2) .. +7 of a
+// 32x32 tile hold (acc_row), so a converted accumulator and this fragment agree on the reduced index
+struct ColFragOffsets {
     int lo[2], hi[2];
     TG_DEVICE explicit ColFragOffsets(int lane) {
         const int g = lane >> 5, blk = (lane >> 4) & 1, i = lane & 15;
@@ -154,12 +108,6 @@ struct ColFragOffsets { // sfrag_cols(tile, kk * 16, dt * 32, lane): rows +kk*16
     }
 };
 
-// ---------------------------------------------------------------------------------------------
-// forward: block = 128 queries (4 waves x 32), key/value tiles of 64 in three LDS stages filled by
-// asynchronous copies issued two tiles ahead; heavy (late) query tiles first.  The tile loop is
-// unrolled by the stage count so every LDS address is a per-lane constant plus an immediate; three
-// resident waves per SIMD overlap one wave's softmax with another's matrix work.
-// ---------------------------------------------------------------------------------------------
 // Block placement.  The work of a causal tile grows with its index and consecutive block ids go to the
 // eight XCDs in turn, so a (tile, head, batch) grid whose tile extent is a multiple of 8 hands one XCD
 // all the heaviest tiles.  Instead each XCD takes every eighth (batch, head) pair with all of that
@@ -191,6 +139,12 @@ TG_DEVICE float halves_sum(float x) {
     return __uint_as_float(both[0]) + __uint_as_float(both[1]);
 }
 
+// ---------------------------------------------------------------------------------------------
+// forward: block = 128 queries (4 waves x 32), key/value tiles of 64 in three LDS stages filled by
+// asynchronous copies issued two tiles ahead; heavy (late) query tiles first.  The tile loop is
+// unrolled by the stage count so every LDS address is a per-lane constant plus an immediate; three
+// resident waves per SIMD overlap one wave's softmax with another's matrix work.
+// ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restrict__ Q,
                                                           const bf16_t *__restrict__ K,
                                                           const bf16_t *__restrict__ V, int ld,
@@ -293,9 +247,10 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restri
                 o[dt] = mfma(vcols.load(vt, kk, dt), pf, o[dt]);
         }
     };
-    for (int j = 0; j < tiles; j += 3) { // tiles is even and block uniform
+    for (int j = 0; j < tiles; j += 3) { // tiles is block uniform
         step(Const<0>{}, j);
-        step(Const<1>{}, j + 1);
+        if (j + 1 < tiles)
+            step(Const<1>{}, j + 1);
         if (j + 2 < tiles)
             step(Const<2>{}, j + 2);
     }
@@ -315,11 +270,13 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restri
         LSE[(size_t(b) * H + h) * T + qrow] = (m + __log2f(l)) * LN2;
 }
 
-// delta[b][h][t] = sum_d dO[t][h*64+d] * O[t][h*64+d]; one 8-lane group per (token, head)
+// delta[b][h][t] = sum_d dO[t][h*64+d] * O[t][h*64+d], and the log-sum-exp rescaled to base 2;
+// one 8-lane group per (token, head)
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *__restrict__ dO, int lddo,
                                                          const bf16_t *__restrict__ O, int ldo,
-                                                         float *__restrict__ delta, int T, int H,
-                                                         int rows) {
+                                                         const float *__restrict__ LSE,
+                                                         float *__restrict__ delta, float *__restrict__ lse2,
+                                                         int T, int H, int rows) {
     const int idx = blockIdx.x * 32 + (threadIdx.x >> 3), part = threadIdx.x & 7;
     if (idx >= rows * H)
         return;
@@ -335,21 +292,26 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *__restric
     sum += __shfl_xor(sum, 4, 64);
     if (part == 0) {
         const int b = token / T, t = token - b * T;
-        delta[(size_t(b) * H + h) * T + t] = sum;
+        const size_t at = (size_t(b) * H + h) * T + t;
+        delta[at] = sum;
+        lse2[at] = LSE[at] * LOG2E;
     }
 }
 
 // ---------------------------------------------------------------------------------------------
-// dK, dV: block = 128 keys (4 waves x 32), loops over 64-query tiles from the diagonal on.
-// Scores are produced as S[query][key] here: one lane owns one KEY, which is the row index of
-// both outputs.
+// dK, dV: block = 128 keys (4 waves x 32), loops over 64-query tiles from the diagonal on; Q and dO
+// tiles (plus the 64 log-sum-exps and deltas of the tile) arrive by asynchronous copies two tiles
+// ahead.  Scores are produced as S[query][key] here: one lane owns one KEY, which is the row index
+// of both outputs.  The two 32-query halves of a tile are processed one after the other to keep the
+// live accumulators, and with them the register count, down.
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
     const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
-    const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ LSE,
+    const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ lse2,
     const float *__restrict__ delta, bf16_t *__restrict__ dK, bf16_t *__restrict__ dV, int lddq, int T,
     int H, int pairs, float scale) {
-    __shared__ __align__(16) bf16_t sQ[2][64 * LS], sdO[2][64 * LS];
+    __shared__ __align__(1024) bf16_t stages[3][2][TILE_ELEMS]; // [stage][Q | dO]
+    __shared__ __align__(256) float rows[3][2][64];             // [stage][lse2 | delta]
     const CausalBlock block = causal_block(H, pairs);
     if (!block.live)
         return;
@@ -358,6 +320,20 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
     const int wave_k0 = k0 + wave * 32, krow = wave_k0 + (lane & 31);
     const size_t token0 = size_t(b) * T;
     const float c = scale * LOG2E;
+    const int first = k0 / 64, tiles = T / 64 - first;
+    const bf16_t *qbase = Q + (token0 + first * 64) * ld + h * HD;
+    const bf16_t *gbase = dO + (token0 + first * 64) * lddo + h * HD;
+    const float *row_source = ((wave & 1) ? delta : lse2) + (size_t(b) * H + h) * T + first * 64 + lane;
+    const uint32_t lds0 = lds_address(&stages[0][0][0]), rows0 = lds_address(&rows[0][wave & 1][0]);
+    auto produce = [&](int stage, int j) { // five copies per wave
+        const uint32_t slot = lds0 + uint32_t(stage) * (2 * TILE_ELEMS * 2);
+        tile_copy_async(slot, qbase + size_t(j) * 64 * ld, ld, wave, lane);
+        tile_copy_async(slot + TILE_ELEMS * 2, gbase + size_t(j) * 64 * lddo, lddo, wave, lane);
+        async_copy4(__builtin_amdgcn_readfirstlane(rows0 + uint32_t(stage) * (2 * 64 * 4)), row_source + j * 64);
+    };
+    produce(0, 0);
+    if (tiles > 1)
+        produce(1, 1);
 
     bf16x8 kf[4], vf[4];
     {
@@ -370,25 +346,20 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
         }
     }
     f32x16 dk[2] = {zero16(), zero16()}, dv[2] = {zero16(), zero16()};
-    const float *lse_row = LSE + (size_t(b) * H + h) * T, *delta_row = delta + (size_t(b) * H + h) * T;
+    const RowFragOffsets qrows(lane);
+    const ColFragOffsets qcols(lane);
 
-    const int first = k0 / 64, tiles = T / 64;
-    const bf16_t *qbase = Q + token0 * ld + h * HD, *gbase = dO + token0 * lddo + h * HD;
-    u32x4 qr[2], gr[2];
-    tile_load(qr, qbase + size_t(first) * 64 * ld, ld, tid);
-    tile_load(gr, gbase + size_t(first) * 64 * lddo, lddo, tid);
-    tile_store(qr, sQ[0], tid);
-    tile_store(gr, sdO[0], tid);
-    __syncthreads();
-    for (int j = first; j < tiles; ++j) {
-        const int cur = (j - first) & 1, q0 = j * 64;
-        const bool more = j + 1 < tiles;
-        if (more) {
-            tile_load(qr, qbase + size_t(q0 + 64) * ld, ld, tid);
-            tile_load(gr, gbase + size_t(q0 + 64) * lddo, lddo, tid);
-        }
-        // the two 32-query halves of the tile are processed one after the other to keep the live
-        // accumulators (and with them the register count, hence two resident blocks per CU) down
+    auto step = [&](auto stage_tag, int j) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        if (j + 1 < tiles)
+            wait_vmcnt<5>(); // only tile j+1's copies may still be in flight
+        else
+            wait_vmcnt<0>();
+        __syncthreads(); // tile j visible to every wave; everyone is done with tile j-1's stage
+        if (j + 2 < tiles)
+            produce((STAGE + 2) % 3, j + 2);
+        const bf16_t *qt_tile = stages[STAGE][0], *gt_tile = stages[STAGE][1];
+        const int q0 = (first + j) * 64;
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             const int qh = q0 + qt * 32;
@@ -397,20 +368,20 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
             f32x16 s = zero16(), dp = zero16();
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
-                s = mfma(frag_rows(sQ[cur], qt * 32, ks * 16, lane), kf[ks], s);
-                dp = mfma(frag_rows(sdO[cur], qt * 32, ks * 16, lane), vf[ks], dp);
+                s = mfma(qrows.load(qt_tile, qt, ks), kf[ks], s);
+                dp = mfma(qrows.load(gt_tile, qt, ks), vf[ks], dp);
             }
             const bool diagonal = qh < wave_k0 + 31;
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
-                const int q = qh + 8 * q4 + 4 * g;
-                const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_row + q);
-                const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_row + q);
+                const int at = qt * 32 + 8 * q4 + 4 * g;
+                const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][0][at]);
+                const f32x4 del4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][1][at]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = q4 * 4 + e;
-                    float p = exp2_fast(fmaf(s[r], c, -lse4[e] * LOG2E));
-                    if (diagonal && krow > q + e)
+                    float p = exp2_fast(fmaf(s[r], c, -lse4[e]));
+                    if (diagonal && krow > q0 + at + e)
                         p = 0.f;
                     s[r] = p;
                     dp[r] = p * (dp[r] - del4[e]);
@@ -422,16 +393,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
                 const bf16x8 dsf = acc_to_frag(dp, kk2);
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt) {
-                    dv[dt] = mfma(frag_cols(sdO[cur], qt * 32 + kk2 * 16, dt * 32, lane), pf, dv[dt]);
-                    dk[dt] = mfma(frag_cols(sQ[cur], qt * 32 + kk2 * 16, dt * 32, lane), dsf, dk[dt]);
+                    dv[dt] = mfma(qcols.load(gt_tile, qt * 2 + kk2, dt), pf, dv[dt]);
+                    dk[dt] = mfma(qcols.load(qt_tile, qt * 2 + kk2, dt), dsf, dk[dt]);
                 }
             }
         }
-        if (more) {
-            tile_store(qr, sQ[cur ^ 1], tid);
-            tile_store(gr, sdO[cur ^ 1], tid);
-        }
-        __syncthreads();
+    };
+    for (int j = 0; j < tiles; j += 3) { // tiles is block uniform
+        step(Const<0>{}, j);
+        if (j + 1 < tiles)
+            step(Const<1>{}, j + 1);
+        if (j + 2 < tiles)
+            step(Const<2>{}, j + 2);
     }
     bf16_t *kp = dK + (token0 + krow) * lddq + h * HD + 4 * g;
     bf16_t *vp = dV + (token0 + krow) * lddq + h * HD + 4 * g;
@@ -450,14 +423,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// dQ: block = 128 queries (4 waves x 32), loops over 64-key tiles up to the diagonal.
+// dQ: block = 128 queries (4 waves x 32), loops over 64-key tiles up to the diagonal; K and V tiles
+// arrive by asynchronous copies two tiles ahead; 32-key halves are processed in turn.
 // ---------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
+__global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
     const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
-    const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ LSE,
+    const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ lse2,
     const float *__restrict__ delta, bf16_t *__restrict__ dQ, int lddq, int T, int H, int pairs,
     float scale) {
-    __shared__ __align__(16) bf16_t sK[2][64 * LS], sV[2][64 * LS];
+    __shared__ __align__(1024) bf16_t stages[3][2][TILE_ELEMS]; // [stage][K | V]
     const CausalBlock block = causal_block(H, pairs);
     if (!block.live)
         return;
@@ -466,6 +440,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
     const int wave_q0 = q0 + wave * 32, qrow = wave_q0 + (lane & 31);
     const size_t token0 = size_t(b) * T;
     const float c = scale * LOG2E;
+    const int tiles = (q0 + 128) / 64;
+    const int my_tiles = wave_q0 / 64 + 1;
+    const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
+    const uint32_t lds0 = lds_address(&stages[0][0][0]);
+    auto produce = [&](int stage, int j) {
+        const uint32_t slot = lds0 + uint32_t(stage) * (2 * TILE_ELEMS * 2);
+        tile_copy_async(slot, kbase + size_t(j) * 64 * ld, ld, wave, lane);
+        tile_copy_async(slot + TILE_ELEMS * 2, vbase + size_t(j) * 64 * ld, ld, wave, lane);
+    };
+    produce(0, 0);
+    if (tiles > 1)
+        produce(1, 1);
 
     bf16x8 qf[4], gf[4];
     {
@@ -477,57 +463,58 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(
             gf[ks] = *reinterpret_cast<const bf16x8 *>(gp + ks * 16);
         }
     }
-    const float lse2 = LSE[(size_t(b) * H + h) * T + qrow] * LOG2E;
+    const float lse = lse2[(size_t(b) * H + h) * T + qrow];
     const float del = delta[(size_t(b) * H + h) * T + qrow];
     f32x16 dq[2] = {zero16(), zero16()};
+    const RowFragOffsets krows(lane);
+    const ColFragOffsets kcols(lane);
 
-    const int tiles = (q0 + 128) / 64;
-    const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
-    u32x4 kr[2], vr[2];
-    tile_load(kr, kbase, ld, tid);
-    tile_load(vr, vbase, ld, tid);
-    tile_store(kr, sK[0], tid);
-    tile_store(vr, sV[0], tid);
-    __syncthreads();
-    for (int j = 0; j < tiles; ++j) {
-        const int cur = j & 1, kv0 = j * 64;
-        const bool more = j + 1 < tiles;
-        if (more) {
-            tile_load(kr, kbase + size_t(kv0 + 64) * ld, ld, tid);
-            tile_load(vr, vbase + size_t(kv0 + 64) * ld, ld, tid);
-        }
-        if (kv0 <= wave_q0 + 31) {
-            f32x16 s[2] = {zero16(), zero16()}, dp[2] = {zero16(), zero16()};
+    auto step = [&](auto stage_tag, int j) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        if (j + 1 < tiles)
+            wait_vmcnt<4>();
+        else
+            wait_vmcnt<0>();
+        __syncthreads();
+        if (j + 2 < tiles)
+            produce((STAGE + 2) % 3, j + 2);
+        if (j >= my_tiles)
+            return;
+        const bf16_t *kt = stages[STAGE][0], *vt = stages[STAGE][1];
+        const int kv0 = j * 64;
+        const bool diagonal = kv0 + 63 > wave_q0;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
+        for (int mt = 0; mt < 2; ++mt) {
+            if (kv0 + mt * 32 > wave_q0 + 31) // every key of this half follows this wave's queries
+                continue;
+            f32x16 s = zero16(), dp = zero16();
 #pragma unroll
-                for (int mt = 0; mt < 2; ++mt) {
-                    s[mt] = mfma(frag_rows(sK[cur], mt * 32, ks * 16, lane), qf[ks], s[mt]);
-                    dp[mt] = mfma(frag_rows(sV[cur], mt * 32, ks * 16, lane), gf[ks], dp[mt]);
-                }
-            const bool diagonal = kv0 + 63 > wave_q0;
+            for (int ks = 0; ks < 4; ++ks) {
+                s = mfma(krows.load(kt, mt, ks), qf[ks], s);
+                dp = mfma(krows.load(vt, mt, ks), gf[ks], dp);
+            }
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
+            for (int r = 0; r < 16; ++r) {
+                float p = exp2_fast(fmaf(s[r], c, -lse));
+                if (diagonal && kv0 + mt * 32 + acc_row(r, g) > qrow)
+                    p = 0.f;
+                dp[r] = p * (dp[r] - del);
+            }
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float p = exp2_fast(fmaf(s[mt][r], c, -lse2));
-                    if (diagonal && kv0 + mt * 32 + acc_row(r, g) > qrow)
-                        p = 0.f;
-                    dp[mt][r] = p * (dp[mt][r] - del);
-                }
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                const bf16x8 dsf = acc_to_frag(dp[kk >> 1], kk & 1);
+            for (int kk2 = 0; kk2 < 2; ++kk2) {
+                const bf16x8 dsf = acc_to_frag(dp, kk2);
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt)
-                    dq[dt] = mfma(frag_cols(sK[cur], kk * 16, dt * 32, lane), dsf, dq[dt]);
+                    dq[dt] = mfma(kcols.load(kt, mt * 2 + kk2, dt), dsf, dq[dt]);
             }
         }
-        if (more) {
-            tile_store(kr, sK[cur ^ 1], tid);
-            tile_store(vr, sV[cur ^ 1], tid);
-        }
-        __syncthreads();
+    };
+    for (int j = 0; j < tiles; j += 3) { // tiles is block uniform
+        step(Const<0>{}, j);
+        if (j + 1 < tiles)
+            step(Const<1>{}, j + 1);
+        if (j + 2 < tiles)
+            step(Const<2>{}, j + 2);
     }
     bf16_t *qp = dQ + (token0 + qrow) * lddq + h * HD + 4 * g;
 #pragma unroll
@@ -572,7 +559,7 @@ extern "C" int tgk_attn_fwd(hipStream_t stream, int B, int H, int T, int hd, con
 }
 
 extern "C" size_t tgk_attn_bwd_workspace(int B, int H, int T) {
-    return size_t(B) * H * T * sizeof(float);
+    return 2 * size_t(B) * H * T * sizeof(float); // delta, and the log-sum-exp in base 2
 }
 
 extern "C" int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
@@ -594,14 +581,14 @@ extern "C" int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, con
         require(workspace && workspace_bytes >= tgk_attn_bwd_workspace(B, H, T) &&
                     !(reinterpret_cast<uintptr_t>(workspace) & 15),
                 "attention backward: workspace too small (see tgk_attn_bwd_workspace)");
-        float *delta = static_cast<float *>(workspace);
+        float *delta = static_cast<float *>(workspace), *lse2 = delta + size_t(B) * H * T;
         const int rows = B * T;
         hipLaunchKernelGGL(attn_delta_kernel, dim3((rows * H + 31) / 32), dim3(256), 0, stream, dO, lddo, O,
-                           ldo, delta, T, H, rows);
+                           ldo, lse, delta, lse2, T, H, rows);
         const dim3 grid(causal_grid(T / 128, B * H));
-        hipLaunchKernelGGL(attn_bwd_dkdv_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse, delta,
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse2, delta,
                            dK, dV, lddq, T, H, B * H, scale);
-        hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse, delta,
+        hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse2, delta,
                            dQ, lddq, T, H, B * H, scale);
         check_hip(hipGetLastError(), "attention backward launch: ");
     });

@@ -82,6 +82,10 @@ TG_DEVICE float wave_max(float x) {
 TG_DEVICE void async_copy16(uint32_t lds_base, const void *global) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(global) : "memory");
 }
+// the 4-byte form: lane l lands at lds_base + 4*l
+TG_DEVICE void async_copy4(uint32_t lds_base, const void *global) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(global) : "memory");
+}
 template <int N> TG_DEVICE void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
