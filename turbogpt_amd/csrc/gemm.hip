@@ -27,11 +27,14 @@ namespace {
 
 enum EpilogueMode { EPI_PLAIN = 0, EPI_RESIDUAL = 1, EPI_GELU = 2, EPI_GELU_BWD = 3 };
 
-// Epilogues work on 4 consecutive n of one m.  An epilogue that needs a second input (residual,
-// saved pre-activation) declares AUX: the kernel fetches those 8 bytes two k-tiles before the end
-// of the reduction, so the epilogue does not wait on memory.
+// An accumulator lane holds 4 consecutive n of one m per register quad.  A plain epilogue (fp32
+// outputs) stores from that layout.  A STAGED epilogue has the kernel round each 32x32 tile to bf16 and
+// transpose it through a wave-private LDS buffer, and then works on 8 consecutive n of one row per
+// lane: one load / store instruction covers 16 rows x 64 contiguous bytes instead of 32 rows x 16
+// bytes.  Its second input (residual, saved pre-activation) is fetched in that row layout two k-tiles
+// before the end of the reduction, so the epilogue does not wait on memory.
 struct EpilogueBf16 {
-    static constexpr bool AUX = true;
+    static constexpr bool STAGED = true;
     bf16_t *out;
     int ld_out;
     const bf16_t *aux; // residual (EPI_RESIDUAL) or saved pre-activation (EPI_GELU_BWD)
@@ -40,44 +43,42 @@ struct EpilogueBf16 {
     int ld_out2;
     int mode;
     TG_DEVICE bool wants_aux() const { return mode == EPI_RESIDUAL || mode == EPI_GELU_BWD; }
-    TG_DEVICE u32x2 load_aux(int m, int n) const {
-        return *reinterpret_cast<const u32x2 *>(aux + size_t(m) * ld_aux + n);
+    TG_DEVICE u32x4 load_aux(int m, int n) const {
+        return *reinterpret_cast<const u32x4 *>(aux + size_t(m) * ld_aux + n);
     }
-    TG_DEVICE void operator()(int m, int n, const float (&v)[4], u32x2 a, int) const {
-        u32x2 packed;
+    // y: the bf16-rounded accumulators of row m, columns n .. n+7
+    TG_DEVICE void finish(int m, int n, u32x4 y, u32x4 a) const {
         if (mode == EPI_RESIDUAL) {
-            // y = RN(RN(acc) + residual): the bf16 add of cuda/mma.cuh:95-97
-            packed.x = pack_bf16(round_bf16(v[0]) + bf16_lo(a.x), round_bf16(v[1]) + bf16_hi(a.x));
-            packed.y = pack_bf16(round_bf16(v[2]) + bf16_lo(a.y), round_bf16(v[3]) + bf16_hi(a.y));
+            // RN(RN(acc) + residual): the bf16 add of cuda/mma.cuh:95-97
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                y[e] = pack_bf16(bf16_lo(y[e]) + bf16_lo(a[e]), bf16_hi(y[e]) + bf16_hi(a[e]));
         } else if (mode == EPI_GELU_BWD) {
             // du = RN(RN(acc) * gelu'(u))
-            packed.x = pack_bf16(round_bf16(v[0]) * gelu_grad_f(bf16_lo(a.x)),
-                                 round_bf16(v[1]) * gelu_grad_f(bf16_hi(a.x)));
-            packed.y = pack_bf16(round_bf16(v[2]) * gelu_grad_f(bf16_lo(a.y)),
-                                 round_bf16(v[3]) * gelu_grad_f(bf16_hi(a.y)));
-        } else {
-            packed.x = pack_bf16(v[0], v[1]);
-            packed.y = pack_bf16(v[2], v[3]);
-            if (mode == EPI_GELU) {
-                u32x2 g;
-                g.x = pack_bf16(gelu_f(bf16_lo(packed.x)), gelu_f(bf16_hi(packed.x)));
-                g.y = pack_bf16(gelu_f(bf16_lo(packed.y)), gelu_f(bf16_hi(packed.y)));
-                *reinterpret_cast<u32x2 *>(out2 + size_t(m) * ld_out2 + n) = g;
-            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                y[e] = pack_bf16(bf16_lo(y[e]) * gelu_grad_f(bf16_lo(a[e])),
+                                 bf16_hi(y[e]) * gelu_grad_f(bf16_hi(a[e])));
+        } else if (mode == EPI_GELU) {
+            u32x4 g;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                g[e] = pack_bf16(gelu_f(bf16_lo(y[e])), gelu_f(bf16_hi(y[e])));
+            *reinterpret_cast<u32x4 *>(out2 + size_t(m) * ld_out2 + n) = g;
         }
-        *reinterpret_cast<u32x2 *>(out + size_t(m) * ld_out + n) = packed;
+        *reinterpret_cast<u32x4 *>(out + size_t(m) * ld_out + n) = y;
     }
 };
 
 struct EpilogueF32 {
-    static constexpr bool AUX = false;
+    static constexpr bool STAGED = false;
     float *out;
     int ld_out;
     size_t split_stride; // elements between split-K slabs
     int accumulate;      // only honoured when there is a single split
     TG_DEVICE bool wants_aux() const { return false; }
-    TG_DEVICE u32x2 load_aux(int, int) const { return u32x2{0, 0}; }
-    TG_DEVICE void operator()(int m, int n, const float (&v)[4], u32x2, int split) const {
+    TG_DEVICE u32x4 load_aux(int, int) const { return u32x4{0, 0, 0, 0}; }
+    TG_DEVICE void operator()(int m, int n, const float (&v)[4], int split) const {
         f32x4 *p = reinterpret_cast<f32x4 *>(out + split * split_stride + size_t(m) * ld_out + n);
         f32x4 value = {v[0], v[1], v[2], v[3]};
         if (accumulate)
@@ -150,8 +151,9 @@ template <int ROWS, bool KC> struct TileOf;
 template <int ROWS> struct TileOf<ROWS, true> { using type = TileKC<ROWS>; };
 template <int ROWS> struct TileOf<ROWS, false> { using type = TileKS<ROWS>; };
 
-template <int BM, int BN, int S> constexpr size_t lds_bytes() {
-    return size_t(S) * (BM + BN) * 64;
+constexpr int STAGING = 4 * 2048; // a 32 x 32 bf16 tile per wave for the row-coalescing epilogue
+template <int BM, int BN, int S, class Epilogue> constexpr size_t lds_bytes() {
+    return size_t(S) * (BM + BN) * 64 + (Epilogue::STAGED ? STAGING : 0);
 }
 
 // C[m][n] = sum_k A(m,k) B(n,k).  A k-contiguous: A[m][k] (lda); k-strided: A[k][m] (lda).  Same for B.
@@ -278,18 +280,20 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
                 for (int r = 0; r < 16; ++r)
                     acc[i][j][r] = 0.f;
         const int out_m = m0 + wm + (lane & 31), out_n = n0 + wn + (lane >> 5) * 4;
-        u32x2 aux[Epilogue::AUX ? FM : 1][Epilogue::AUX ? FN : 1][4];
+        // row layout of the staged epilogue: this lane finishes rows get_row and get_row + 16, 8 columns
+        const int get_row = lane >> 2, get_chunk = lane & 3;
+        u32x4 aux[Epilogue::STAGED ? FM : 1][Epilogue::STAGED ? FN : 1][2];
         const int aux_at = nk > 2 ? nk - 2 : 0;
         for (int kt = 0; kt < nk; ++kt) {
-            if (Epilogue::AUX && kt == aux_at && epilogue.wants_aux()) {
+            if (Epilogue::STAGED && kt == aux_at && epilogue.wants_aux()) {
 #pragma unroll
                 for (int i = 0; i < FM; ++i)
 #pragma unroll
                     for (int j = 0; j < FN; ++j)
 #pragma unroll
-                        for (int q = 0; q < 4; ++q)
-                            aux[Epilogue::AUX ? i : 0][Epilogue::AUX ? j : 0][q] =
-                                epilogue.load_aux(out_m + i * 32, out_n + j * 32 + q * 8);
+                        for (int half = 0; half < 2; ++half)
+                            aux[Epilogue::STAGED ? i : 0][Epilogue::STAGED ? j : 0][half] = epilogue.load_aux(
+                                m0 + wm + i * 32 + get_row + half * 16, n0 + wn + j * 32 + get_chunk * 8);
             }
             // in flight now: the stage being consumed (landed), then inflight-1 younger ones; the next one
             // must land too
@@ -313,17 +317,42 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[j], af1[i], acc[i][j], 0, 0, 0);
             c_slot = next_slot;
         }
+        if constexpr (Epilogue::STAGED) {
+            // wave-private buffer: 32 rows of 64 bytes, 16-byte chunk c of row r at c ^ ((r >> 2) & 3).
+            // LDS operations of one wave execute in order, so no barrier is needed around it.
+            unsigned char *mine = smem + S * STAGE + wave * 2048;
+            const int row = lane & 31;
+            unsigned char *put = mine + row * 64 + (lane >> 5) * 8;
+            const int put_swizzle = (row >> 2) & 3;
+            // rows r and r + 16 share a swizzle term, so the second half is 1 KiB further on
+            const unsigned char *get = mine + get_row * 64 + ((get_chunk ^ ((get_row >> 2) & 3)) << 4);
 #pragma unroll
-        for (int i = 0; i < FM; ++i)
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
+                for (int j = 0; j < FN; ++j) {
+                    const int m = m0 + wm + i * 32 + get_row, n = n0 + wn + j * 32 + get_chunk * 8;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
-                                        acc[i][j][q * 4 + 3]};
-                    epilogue(out_m + i * 32, out_n + j * 32 + q * 8, v,
-                             aux[Epilogue::AUX ? i : 0][Epilogue::AUX ? j : 0][q], split);
+                    for (int q = 0; q < 4; ++q) {
+                        u32x2 packed;
+                        packed.x = pack_bf16(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
+                        packed.y = pack_bf16(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+                        *reinterpret_cast<u32x2 *>(put + ((q ^ put_swizzle) << 4)) = packed;
+                    }
+                    epilogue.finish(m, n, *reinterpret_cast<const u32x4 *>(get), aux[i][j][0]);
+                    epilogue.finish(m + 16, n, *reinterpret_cast<const u32x4 *>(get + 1024), aux[i][j][1]);
                 }
+        } else {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                                            acc[i][j][q * 4 + 3]};
+                        epilogue(out_m + i * 32, out_n + j * 32 + q * 8, v, split);
+                    }
+        }
     }
     wait_vmcnt<0>();
 }
@@ -386,7 +415,7 @@ template <int BM, int BN, int S, bool AKC, bool BKC, class Epilogue>
 void launch_gemm(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N,
                  int K, int splits, int max_blocks, const Epilogue &epilogue) {
     auto kernel = gemm_kernel<BM, BN, S, AKC, BKC, Epilogue>;
-    constexpr size_t lds = lds_bytes<BM, BN, S>();
+    constexpr size_t lds = lds_bytes<BM, BN, S, Epilogue>();
     static bool configured = false;
     if (!configured) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
