@@ -449,7 +449,7 @@ TG_API int tg_blocks(Engine *e) {
     return e->compute_units;
 }
 TG_API int tg_shared_bytes(Engine *) {
-    return 3 * (128 + 192) * 64 + 4 * 2048; // the 128x192 GEMM: three 32-k stages plus the epilogue's staging tiles
+    return 3 * (128 + 192) * 64 + 4 * 4096; // the 128x192 GEMM: three 32-k stages plus the epilogue's fp32 staging tiles
 }
 TG_API int tg_synchronize(Engine *e) {
     return guarded([&] {

@@ -34,7 +34,7 @@ enum EpilogueMode { EPI_PLAIN = 0, EPI_RESIDUAL = 1, EPI_GELU = 2, EPI_GELU_BWD 
 // bytes.  Its second input (residual, saved pre-activation) is fetched in that row layout two k-tiles
 // before the end of the reduction, so the epilogue does not wait on memory.
 struct EpilogueBf16 {
-    static constexpr bool STAGED = true;
+    static constexpr bool BF16 = true;
     bf16_t *out;
     int ld_out;
     const bf16_t *aux; // residual (EPI_RESIDUAL) or saved pre-activation (EPI_GELU_BWD)
@@ -70,17 +70,18 @@ struct EpilogueBf16 {
     }
 };
 
+// fp32 outputs (weight gradients, split-K slabs): tiles go through the same kind of wave-private LDS
+// buffer untouched, and a lane finishes 4 consecutive n - 8 lanes cover a 128-byte row piece.
 struct EpilogueF32 {
-    static constexpr bool STAGED = false;
+    static constexpr bool BF16 = false;
     float *out;
     int ld_out;
     size_t split_stride; // elements between split-K slabs
     int accumulate;      // only honoured when there is a single split
     TG_DEVICE bool wants_aux() const { return false; }
     TG_DEVICE u32x4 load_aux(int, int) const { return u32x4{0, 0, 0, 0}; }
-    TG_DEVICE void operator()(int m, int n, const float (&v)[4], int split) const {
+    TG_DEVICE void finish(int m, int n, f32x4 value, int split) const {
         f32x4 *p = reinterpret_cast<f32x4 *>(out + split * split_stride + size_t(m) * ld_out + n);
-        f32x4 value = {v[0], v[1], v[2], v[3]};
         if (accumulate)
             value += *p;
         *p = value;
@@ -151,9 +152,9 @@ template <int ROWS, bool KC> struct TileOf;
 template <int ROWS> struct TileOf<ROWS, true> { using type = TileKC<ROWS>; };
 template <int ROWS> struct TileOf<ROWS, false> { using type = TileKS<ROWS>; };
 
-constexpr int STAGING = 4 * 2048; // a 32 x 32 bf16 tile per wave for the row-coalescing epilogue
+// pipeline stages plus one 32 x 32 output tile per wave for the row-coalescing epilogue
 template <int BM, int BN, int S, class Epilogue> constexpr size_t lds_bytes() {
-    return size_t(S) * (BM + BN) * 64 + (Epilogue::STAGED ? STAGING : 0);
+    return size_t(S) * (BM + BN) * 64 + 4 * (Epilogue::BF16 ? 2048 : 4096);
 }
 
 // C[m][n] = sum_k A(m,k) B(n,k).  A k-contiguous: A[m][k] (lda); k-strided: A[k][m] (lda).  Same for B.
@@ -279,20 +280,19 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     acc[i][j][r] = 0.f;
-        const int out_m = m0 + wm + (lane & 31), out_n = n0 + wn + (lane >> 5) * 4;
         // row layout of the staged epilogue: this lane finishes rows get_row and get_row + 16, 8 columns
         const int get_row = lane >> 2, get_chunk = lane & 3;
-        u32x4 aux[Epilogue::STAGED ? FM : 1][Epilogue::STAGED ? FN : 1][2];
+        u32x4 aux[Epilogue::BF16 ? FM : 1][Epilogue::BF16 ? FN : 1][2];
         const int aux_at = nk > 2 ? nk - 2 : 0;
         for (int kt = 0; kt < nk; ++kt) {
-            if (Epilogue::STAGED && kt == aux_at && epilogue.wants_aux()) {
+            if (Epilogue::BF16 && kt == aux_at && epilogue.wants_aux()) {
 #pragma unroll
                 for (int i = 0; i < FM; ++i)
 #pragma unroll
                     for (int j = 0; j < FN; ++j)
 #pragma unroll
                         for (int half = 0; half < 2; ++half)
-                            aux[Epilogue::STAGED ? i : 0][Epilogue::STAGED ? j : 0][half] = epilogue.load_aux(
+                            aux[Epilogue::BF16 ? i : 0][Epilogue::BF16 ? j : 0][half] = epilogue.load_aux(
                                 m0 + wm + i * 32 + get_row + half * 16, n0 + wn + j * 32 + get_chunk * 8);
             }
             // in flight now: the stage being consumed (landed), then inflight-1 younger ones; the next one
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bf1[j], af1[i], acc[i][j], 0, 0, 0);
             c_slot = next_slot;
         }
-        if constexpr (Epilogue::STAGED) {
+        if constexpr (Epilogue::BF16) {
             // wave-private buffer: 32 rows of 64 bytes, 16-byte chunk c of row r at c ^ ((r >> 2) & 3).
             // LDS operations of one wave execute in order, so no barrier is needed around it.
             unsigned char *mine = smem + S * STAGE + wave * 2048;
@@ -342,16 +342,29 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
                     epilogue.finish(m + 16, n, *reinterpret_cast<const u32x4 *>(get + 1024), aux[i][j][1]);
                 }
         } else {
+            // wave-private buffer: 32 rows of 128 bytes, 16-byte chunk c of row r at c ^ ((r >> 1) & 7)
+            unsigned char *mine = smem + S * STAGE + wave * 4096;
+            const int row = lane & 31;
+            unsigned char *put = mine + row * 128;
+            const int put_swizzle = (row >> 1) & 7, g = lane >> 5;
+            const int first_row = lane >> 3, chunk = lane & 7;
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
+                for (int j = 0; j < FN; ++j) {
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const float v[4] = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
-                                            acc[i][j][q * 4 + 3]};
-                        epilogue(out_m + i * 32, out_n + j * 32 + q * 8, v, split);
+                        const f32x4 v = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                                         acc[i][j][q * 4 + 3]};
+                        *reinterpret_cast<f32x4 *>(put + (((2 * q + g) ^ put_swizzle) << 4)) = v;
                     }
+#pragma unroll
+                    for (int part = 0; part < 4; ++part) {
+                        const int r = first_row + part * 8;
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(mine + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4));
+                        epilogue.finish(m0 + wm + i * 32 + r, n0 + wn + j * 32 + chunk * 4, v, split);
+                    }
+                }
         }
     }
     wait_vmcnt<0>();
