@@ -11,9 +11,10 @@
 // no cross-lane movement.  The operand that must then be read "k-strided" (V for P.V, K for dS.K,
 // Q and dO for the dK/dV products) is fetched with the transposing LDS read ds_read_b64_tr_b16.
 //
-// backward = three launches: delta = rowsum(dO o O); dK/dV (one block per 128 keys, loops over
-// query tiles); dQ (one block per 128 queries, loops over key tiles).  No atomics: every output
-// element has one owner and a fixed summation order, so results are bit-reproducible.
+// backward = two launches: dQ (one block per 128 queries, loops over key tiles; it also computes
+// delta = rowsum(dO o O) for its queries), then dK/dV (one block per 128 keys, loops over query
+// tiles).  No atomics: every output element has one owner and a fixed summation order, so results
+// are bit-reproducible.
 #include "common.h"
 #include "../../include/tgk_kernels.h"
 
@@ -270,34 +271,6 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restri
         LSE[(size_t(b) * H + h) * T + qrow] = (m + __log2f(l)) * LN2;
 }
 
-// delta[b][h][t] = sum_d dO[t][h*64+d] * O[t][h*64+d], and the log-sum-exp rescaled to base 2;
-// one 8-lane group per (token, head)
-__global__ __launch_bounds__(256) void attn_delta_kernel(const bf16_t *__restrict__ dO, int lddo,
-                                                         const bf16_t *__restrict__ O, int ldo,
-                                                         const float *__restrict__ LSE,
-                                                         float *__restrict__ delta, float *__restrict__ lse2,
-                                                         int T, int H, int rows) {
-    const int idx = blockIdx.x * 32 + (threadIdx.x >> 3), part = threadIdx.x & 7;
-    if (idx >= rows * H)
-        return;
-    const int token = idx / H, h = idx - token * H;
-    const u32x4 a = *reinterpret_cast<const u32x4 *>(dO + size_t(token) * lddo + h * HD + part * 8);
-    const u32x4 o = *reinterpret_cast<const u32x4 *>(O + size_t(token) * ldo + h * HD + part * 8);
-    float sum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        sum += bf16_lo(a[i]) * bf16_lo(o[i]) + bf16_hi(a[i]) * bf16_hi(o[i]);
-    sum += __shfl_xor(sum, 1, 64);
-    sum += __shfl_xor(sum, 2, 64);
-    sum += __shfl_xor(sum, 4, 64);
-    if (part == 0) {
-        const int b = token / T, t = token - b * T;
-        const size_t at = (size_t(b) * H + h) * T + t;
-        delta[at] = sum;
-        lse2[at] = LSE[at] * LOG2E;
-    }
-}
-
 // ---------------------------------------------------------------------------------------------
 // dK, dV: block = 128 keys (4 waves x 32), loops over 64-query tiles from the diagonal on; Q and dO
 // tiles (plus the 64 log-sum-exps and deltas of the tile) arrive by asynchronous copies two tiles
@@ -428,9 +401,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
     const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V, int ld,
-    const bf16_t *__restrict__ dO, int lddo, const float *__restrict__ lse2,
-    const float *__restrict__ delta, bf16_t *__restrict__ dQ, int lddq, int T, int H, int pairs,
-    float scale) {
+    const bf16_t *__restrict__ dO, int lddo, const bf16_t *__restrict__ O, int ldo,
+    const float *__restrict__ LSE, float *__restrict__ lse2_out, float *__restrict__ delta_out,
+    bf16_t *__restrict__ dQ, int lddq, int T, int H, int pairs, float scale) {
     __shared__ __align__(1024) bf16_t stages[3][2][TILE_ELEMS]; // [stage][K | V]
     const CausalBlock block = causal_block(H, pairs);
     if (!block.live)
@@ -463,8 +436,26 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
             gf[ks] = *reinterpret_cast<const bf16x8 *>(gp + ks * 16);
         }
     }
-    const float lse = lse2[(size_t(b) * H + h) * T + qrow];
-    const float del = delta[(size_t(b) * H + h) * T + qrow];
+    // delta = rowsum(dO o O) and the log-sum-exp in base 2, for this block's own queries; also left in
+    // memory for the dK/dV kernel, which runs after this one
+    float del = 0.f;
+    {
+        const bf16_t *op = O + (token0 + qrow) * ldo + h * HD + g * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x8 of = *reinterpret_cast<const bf16x8 *>(op + ks * 16);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                del += float(gf[ks][e]) * float(of[e]);
+        }
+        del = halves_sum(del);
+    }
+    const size_t row_at = (size_t(b) * H + h) * T + qrow;
+    const float lse = LSE[row_at] * LOG2E;
+    if (g == 0) {
+        delta_out[row_at] = del;
+        lse2_out[row_at] = lse;
+    }
     f32x16 dq[2] = {zero16(), zero16()};
     const RowFragOffsets krows(lane);
     const ColFragOffsets kcols(lane);
@@ -582,14 +573,11 @@ extern "C" int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, con
                     !(reinterpret_cast<uintptr_t>(workspace) & 15),
                 "attention backward: workspace too small (see tgk_attn_bwd_workspace)");
         float *delta = static_cast<float *>(workspace), *lse2 = delta + size_t(B) * H * T;
-        const int rows = B * T;
-        hipLaunchKernelGGL(attn_delta_kernel, dim3((rows * H + 31) / 32), dim3(256), 0, stream, dO, lddo, O,
-                           ldo, lse, delta, lse2, T, H, rows);
         const dim3 grid(causal_grid(T / 128, B * H));
+        hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, O, ldo, lse,
+                           lse2, delta, dQ, lddq, T, H, B * H, scale);
         hipLaunchKernelGGL(attn_bwd_dkdv_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse2, delta,
                            dK, dV, lddq, T, H, B * H, scale);
-        hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse2, delta,
-                           dQ, lddq, T, H, B * H, scale);
         check_hip(hipGetLastError(), "attention backward launch: ");
     });
 }
