@@ -22,7 +22,7 @@ def hilo(orc, w):
     return dev(hi.view(np.int16)), dev(lo.view(np.int16))
 
 
-@pytest.mark.parametrize("B,T,D", [(2, 128, 256), (3, 64, 768), (9, 256, 128)])
+@pytest.mark.parametrize("B,T,D", [(2, 128, 256), (3, 64, 768), (9, 256, 128), (2, 50, 64), (5, 1000, 320)])
 def test_embedding_forward_and_backward(orc, B, T, D):
     lib = library()
     rng = np.random.default_rng(B + T + D)

@@ -92,6 +92,18 @@ __global__ __launch_bounds__(256) void embed_bwd_fold_kernel(const float *__rest
         sum += partial[size_t(s) * count + i];
     dtable[i] = accumulate ? dtable[i] + sum : sum;
 }
+// onehot[t][v] = (x[t] == v) in bf16; one thread writes 8 columns
+__global__ __launch_bounds__(256) void onehot_kernel(const uint8_t *__restrict__ x, bf16_t *__restrict__ onehot,
+                                                     int rows) {
+    const size_t total = size_t(rows) * 32;
+    for (size_t i = blockIdx.x * size_t(256) + threadIdx.x; i < total; i += size_t(gridDim.x) * 256) {
+        const int t = int(i >> 5), c0 = int(i & 31) * 8, hot = int(x[t]) - c0;
+        u32x4 v = {0, 0, 0, 0};
+        if (hot >= 0 && hot < 8)
+            v[hot >> 1] = (hot & 1) ? 0x3f800000u : 0x00003f80u; // bf16 1.0 in the high / low half
+        *reinterpret_cast<u32x4 *>(onehot + size_t(t) * 256 + c0) = v;
+    }
+}
 // dPositions[p][c] = sum over sequences b of dh[b*T + p][c]
 __global__ __launch_bounds__(256) void embed_bwd_positions_kernel(const bf16_t *__restrict__ dh,
                                                                   float *__restrict__ dpos, int B, int T,
@@ -520,9 +532,20 @@ extern "C" int tgk_embed_fwd(hipStream_t stream, int rows, int T, int D, const u
     });
 }
 
+// The token-table gradient is a product: dTable[v][c] = sum_t onehot[t][v] dh[t][c], i.e. the weight-
+// gradient GEMM with the one-hot matrix as its "dY" (exact in bf16).  Shapes that GEMM does not take
+// go through the LDS-table kernels above.
+static bool embed_bwd_as_gemm(int rows, int D) {
+    return rows % 32 == 0 && D % 128 == 0;
+}
+static size_t onehot_bytes(int rows) {
+    return size_t(rows) * 256 * sizeof(bf16_t);
+}
 extern "C" size_t tgk_embed_bwd_workspace(int rows, int D) {
     if (rows <= 0 || D <= 0)
         return 0;
+    if (embed_bwd_as_gemm(rows, D))
+        return onehot_bytes(rows) + tgk_gemm_wgrad_workspace(rows, 256, D);
     return size_t((rows + EMBED_SEGMENT - 1) / EMBED_SEGMENT) * 256 * D * sizeof(float);
 }
 extern "C" int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab, const uint8_t *x,
@@ -533,14 +556,26 @@ extern "C" int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab,
         require(vocab == 256, "embed_bwd: vocabulary must be 256 (byte tokens)");
         require(x && dh && dtable && dpositions, "embed_bwd: missing operand");
         const int rows = B * T, segments = (rows + EMBED_SEGMENT - 1) / EMBED_SEGMENT;
-        require(workspace && workspace_bytes >= tgk_embed_bwd_workspace(rows, D),
+        require(workspace && workspace_bytes >= tgk_embed_bwd_workspace(rows, D) &&
+                    !(reinterpret_cast<uintptr_t>(workspace) & 15),
                 "embed_bwd: workspace too small (see tgk_embed_bwd_workspace)");
-        float *partial = static_cast<float *>(workspace);
-        hipLaunchKernelGGL(embed_bwd_partial_kernel, dim3(D / 64, segments), dim3(64), 0, stream, x, dh, partial,
-                           rows, D);
-        const size_t count = size_t(256) * D;
-        hipLaunchKernelGGL(embed_bwd_fold_kernel, dim3(unsigned((count + 255) / 256)), dim3(256), 0, stream, partial,
-                           segments, dtable, count, accumulate);
+        if (embed_bwd_as_gemm(rows, D)) {
+            bf16_t *onehot = static_cast<bf16_t *>(workspace);
+            hipLaunchKernelGGL(onehot_kernel, dim3(grid_for(size_t(rows) * 32, 256)), dim3(256), 0, stream, x,
+                               onehot, rows);
+            check_hip(hipGetLastError(), "embed_bwd launch: ");
+            if (tgk_gemm_wgrad(stream, rows, 256, D, onehot, 256, dh, D, dtable, D, accumulate,
+                               static_cast<char *>(workspace) + onehot_bytes(rows),
+                               workspace_bytes - onehot_bytes(rows)) != 0)
+                throw std::runtime_error("embed_bwd: " + tg_last_error);
+        } else {
+            float *partial = static_cast<float *>(workspace);
+            hipLaunchKernelGGL(embed_bwd_partial_kernel, dim3(D / 64, segments), dim3(64), 0, stream, x, dh,
+                               partial, rows, D);
+            const size_t count = size_t(256) * D;
+            hipLaunchKernelGGL(embed_bwd_fold_kernel, dim3(unsigned((count + 255) / 256)), dim3(256), 0, stream,
+                               partial, segments, dtable, count, accumulate);
+        }
         hipLaunchKernelGGL(embed_bwd_positions_kernel, dim3(grid_for(size_t(T) * D, 256)), dim3(256), 0, stream,
                            dh, dpositions, B, T, D, accumulate);
         check_hip(hipGetLastError(), "embed_bwd launch: ");
