@@ -24,6 +24,11 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 D, L, H, T, B, V = 768, 12, 12, 1024, 16, 256
 F = 4 * D
 M = B * T
+# mean over the four projection shapes of 2 * (M*K + N*K + M*N) bytes: operands read and the result written once
+ALGORITHMIC_BYTES_PER_LAUNCH = sum(2 * (M * k + n * k + M * n) for n, k in
+                                   [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
+# HBM bytes per launch of that kernel measured with rocprofv3 counters (profiles/gemm_kc_ks_hbm_traffic.md)
+HBM_TRAFFIC_PER_LAUNCH = 150.5e6
 
 
 def gemm_flops():
@@ -126,12 +131,15 @@ def kernel_sweeps(out):
         y = torch.empty(M, n, device="cuda", dtype=torch.bfloat16)
         dx = torch.empty(M, k, device="cuda", dtype=torch.bfloat16)
         dw = torch.empty(n, k, device="cuda")
+        wt = w.t().contiguous()
         need = lib.tgk_gemm_wgrad_workspace(M, n, k)
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
         flop = 2.0 * M * n * k
         runs = {
             "fwd": lambda: check(lib.tgk_gemm_fwd(stream, M, n, k, x.data_ptr(), k, w.data_ptr(), k, y.data_ptr(), n,
                                                   None, 0, None, 0)),
+            "fwd_t": lambda: check(lib.tgk_gemm_fwd_t(stream, M, n, k, x.data_ptr(), k, wt.data_ptr(), n,
+                                                      y.data_ptr(), n, None, 0, None, 0)),
             "dgrad": lambda: check(lib.tgk_gemm_dgrad(stream, M, n, k, dy.data_ptr(), n, w.data_ptr(), k,
                                                       dx.data_ptr(), k, None, 0)),
             "wgrad": lambda: check(lib.tgk_gemm_wgrad(stream, M, n, k, dy.data_ptr(), n, x.data_ptr(), k,
@@ -167,7 +175,9 @@ def kernel_sweeps(out):
 
 def traffic_probe():
     """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: one plain copy of known size (256 MiB in,
-    256 MiB out: the calibration dispatch) followed by one launch of each forward block projection."""
+    256 MiB out: the calibration dispatch) followed by one launch of each forward block projection
+    (on transposed weights, as the engine runs them) and of each dgrad - the eight uses per layer of
+    the kernel that `roofline` describes."""
     import torch
     from turbogpt_amd.bridge import check, library
     lib = library()
@@ -177,16 +187,23 @@ def traffic_probe():
     torch.cuda.synchronize()
     dst.copy_(src)
     torch.cuda.synchronize()
-    for k, n in [(768, 2304), (768, 768), (768, 3072), (3072, 768)]:
+    shapes = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
+    for k, n in shapes:
         x = torch.randn(M, k, device="cuda").bfloat16()
         w = torch.randn(n, k, device="cuda").bfloat16()
+        wt = w.t().contiguous()
+        dy = torch.randn(M, n, device="cuda").bfloat16()
         y = torch.empty(M, n, device="cuda", dtype=torch.bfloat16)
+        dx = torch.empty(M, k, device="cuda", dtype=torch.bfloat16)
         torch.cuda.synchronize()
-        check(lib.tgk_gemm_fwd(stream, M, n, k, x.data_ptr(), k, w.data_ptr(), k, y.data_ptr(), n, None, 0, None, 0))
+        check(lib.tgk_gemm_fwd_t(stream, M, n, k, x.data_ptr(), k, wt.data_ptr(), n, y.data_ptr(), n, None, 0,
+                                 None, 0))
+        torch.cuda.synchronize()
+        check(lib.tgk_gemm_dgrad(stream, M, n, k, dy.data_ptr(), n, w.data_ptr(), k, dx.data_ptr(), k, None, 0))
         torch.cuda.synchronize()
     print(json.dumps({"probe": "traffic", "copy_bytes_each_way": 1 << 28,
-                      "gemm_fwd_algorithmic_bytes": [2 * (M * k + n * k + M * n) for k, n in
-                                                     [(768, 2304), (768, 768), (768, 3072), (3072, 768)]]}))
+                      "order": "per shape (K, N): forward, then dgrad", "shapes": shapes,
+                      "algorithmic_bytes_per_launch": [2 * (M * k + n * k + M * n) for k, n in shapes]}))
 
 
 def main():
@@ -239,11 +256,14 @@ def main():
         rate = amount / (per_step_ms * 1e-3) / 1e12 if per_step_ms > 0 else 0.0
         classes[name] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // 3,
                          ("tflops" if kind == "flop" else "tb_per_s"): round(rate, 2)}
-    # dominant MFMA kernel: the forward block-projection GEMM (one template instantiation, 4 launches/layer);
-    # traffic: profiles/gemm_fwd_hbm_traffic.md (FETCH_SIZE/WRITE_SIZE runs of --traffic-probe), mean of the 4 shapes
+    # dominant MFMA kernel: gemm_kernel<128,192,3,true,false,EpilogueBf16> - activations k-contiguous,
+    # weights k-strided - which runs the forward block projections (on the transposed weights) and the
+    # dgrads: 8 launches per layer, 96 per step, the same four shapes in both directions.
     fwd_ms, fwd_launches = profile["gemm_fwd"]
+    dgrad_ms, dgrad_launches = profile["gemm_dgrad"]
+    launch_ms = (fwd_ms + dgrad_ms) / (fwd_launches + dgrad_launches)
     flops_per_launch = sum(gemm_flops()) / 4
-    achieved = flops_per_launch / (fwd_ms / fwd_launches * 1e-3) / 1e12
+    achieved = flops_per_launch / (launch_ms * 1e-3) / 1e12
     ms_per_step = seconds / args.steps * 1e3
     result = {
         "metric": "train tokens/sec at d768 L12 T1024 (1 GPU)",
@@ -262,11 +282,15 @@ def main():
                                "ffn=3072 vocab=256, bf16 weights with fp32 masters, AdamW lr 3e-4 betas 0.9/0.95 "
                                "wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
                    "global_batch": B, "seq_len": T, "parameters": params, "parallelism": "single GPU"},
-        "roofline": {"bound": "mfma", "kernel": "gemm_kernel<128,128,true,true,EpilogueBf16> (forward block "
-                     "projections: QKV, attention-out, MLP-up, MLP-down)", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                     "flops_per_launch": flops_per_launch,
-                     "avg_launch_ms": round(fwd_ms / fwd_launches, 5)},
+        "roofline": {"bound": "mfma",
+                     "kernel": "gemm_kernel<128,192,3,true,false,EpilogueBf16> (forward block projections and "
+                               "dgrads: QKV, attention-out, MLP-up, MLP-down)",
+                     "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": HBM_TRAFFIC_PER_LAUNCH,
+                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated; "
+                                     "profiles/gemm_kc_ks_hbm_traffic.md)",
+                     "algorithmic_bytes_per_launch": ALGORITHMIC_BYTES_PER_LAUNCH,
+                     "flops_per_launch": flops_per_launch, "avg_launch_ms": round(launch_ms, 5)},
         "classes": classes,
         # 9.45 TFLOP of algorithmic work per step (attention causal-counted, backward = 2.5 x forward)
         "model_tflops": round((3 * L * sum(gemm_flops()) + 3 * 2.0 * M * V * D +

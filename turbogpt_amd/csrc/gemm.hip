@@ -163,7 +163,7 @@ template <int BM, int BN, int S, class Epilogue> constexpr size_t lds_bytes() {
 template <int BM, int BN, int S, bool AKC, bool BKC, class Epilogue>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__ A, int lda,
                                                     const bf16_t *__restrict__ B, int ldb, int k_tiles,
-                                                    int splits, int tiles_n, int tiles_total,
+                                                    int splits, int tiles_n, int tiles_total, int xcd_cols,
                                                     Epilogue epilogue) {
     using TA = typename TileOf<BM, AKC>::type;
     using TB = typename TileOf<BN, BKC>::type;
@@ -177,14 +177,29 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
     const int items = tiles_total * splits, stride = gridDim.x;
 
-    // item -> (m0, n0, first k-tile, k-tile count); blocks of one XCD get contiguous tiles
+    // item -> (m0, n0, first k-tile, k-tile count).  Consecutive block ids sit on consecutive XCDs, each
+    // with an L2 of its own, so item i belongs to XCD i % 8 and is that XCD's (i / 8)-th item.  The tile
+    // grid is cut into (8 / xcd_cols) x xcd_cols rectangles, one per XCD, walked row-major: an XCD
+    // streams its rows of A once and keeps its columns of B in L2.  (xcd_cols = 1 with split-K items:
+    // every XCD owns a contiguous run of (split, tile).)
     auto locate = [&](int item, int &m0, int &n0, int &kt0, int &nk) {
-        int logical = item;
-        if ((items & 7) == 0)
-            logical = (item & 7) * (items >> 3) + (item >> 3);
-        const int split = logical / tiles_total, tile = logical - split * tiles_total;
-        m0 = (tile / tiles_n) * BM;
-        n0 = (tile % tiles_n) * BN;
+        int split = 0, tile_m, tile_n;
+        if ((items & 7) == 0 && xcd_cols > 1) {
+            const int xcd = item & 7, index = item >> 3;
+            const int cols = tiles_n / xcd_cols, rows = (tiles_total / tiles_n) / (8 / xcd_cols);
+            tile_m = (xcd / xcd_cols) * rows + index / cols;
+            tile_n = (xcd % xcd_cols) * cols + index % cols;
+        } else {
+            int logical = item;
+            if ((items & 7) == 0)
+                logical = (item & 7) * (items >> 3) + (item >> 3);
+            split = logical / tiles_total;
+            const int tile = logical - split * tiles_total;
+            tile_m = tile / tiles_n;
+            tile_n = tile % tiles_n;
+        }
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
         kt0 = split * k_tiles / splits;
         nk = (split + 1) * k_tiles / splits - kt0;
         return split;
@@ -424,6 +439,31 @@ int tile_rows(Tile) { return 128; }
 int tile_cols(Tile t) { return t == TILE_128x128 ? 128 : 192; }
 int resident_blocks(Tile) { return compute_units() * 2; }
 
+// How many column groups to cut the tile grid into for the eight XCDs (see locate()).  Estimated
+// reads beyond L2: every XCD column group streams all of A once; an XCD re-reads its slice of B once
+// per pass over its rows unless the slice stays in its 4 MiB L2 beside the streaming operand.
+int xcd_columns(int tiles_m, int tiles_n, int BM, int BN, int K, int blocks) {
+    if ((tiles_m * tiles_n) % 8)
+        return 1;
+    const double a_bytes = 2.0 * tiles_m * BM * K, b_bytes = 2.0 * tiles_n * BN * K;
+    const int concurrent = blocks / 8 > 0 ? blocks / 8 : 1; // tiles in flight per XCD
+    int best = 1;
+    double best_cost = 0;
+    for (int columns = 1; columns <= 8; columns *= 2) {
+        const int xcd_rows = 8 / columns;
+        if (tiles_n % columns || tiles_m % xcd_rows)
+            continue;
+        const double slice = b_bytes / columns;
+        const int cols = tiles_n / columns, rows = tiles_m / xcd_rows;
+        const int rows_in_flight = concurrent / cols > 0 ? concurrent / cols : 1;
+        const int passes = slice <= 2.5 * 1048576 ? 1 : (rows + rows_in_flight - 1) / rows_in_flight;
+        const double cost = a_bytes * columns + 8 * slice * passes;
+        if (columns == 1 || cost < best_cost)
+            best = columns, best_cost = cost;
+    }
+    return best;
+}
+
 template <int BM, int BN, int S, bool AKC, bool BKC, class Epilogue>
 void launch_gemm(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N,
                  int K, int splits, int max_blocks, const Epilogue &epilogue) {
@@ -436,9 +476,10 @@ void launch_gemm(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, 
                   "gemm LDS size: ");
         configured = true;
     }
-    const int tiles_n = N / BN, tiles = (M / BM) * tiles_n, items = tiles * splits;
-    hipLaunchKernelGGL(kernel, dim3(items < max_blocks ? items : max_blocks), dim3(256), lds, stream, A, lda, B,
-                       ldb, K / BK, splits, tiles_n, tiles, epilogue);
+    const int tiles_m = M / BM, tiles_n = N / BN, tiles = tiles_m * tiles_n, items = tiles * splits;
+    const int blocks = items < max_blocks ? items : max_blocks;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, A, lda, B, ldb, K / BK, splits, tiles_n, tiles,
+                       splits == 1 ? xcd_columns(tiles_m, tiles_n, BM, BN, K, blocks) : 1, epilogue);
     check_hip(hipGetLastError(), "gemm launch: ");
 }
 
