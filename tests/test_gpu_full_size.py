@@ -1,0 +1,88 @@
+"""BASELINE configs[3] (d768 L12 T1024 B16) and configs[4] (d1024 L24 H16 T4096 B4) at full size
+through the tg_* C ABI, checked by properties that do not need the CPU checker at that size:
+bit-exact causality (tests/verify.py:43-50), run-to-run determinism of training, a first loss near
+ln 256 for N(0, 0.02) weights that falls under AdamW, and the flat-gradient identity
+<grad, w> for the scale-free final LayerNorm."""
+import numpy as np
+import pytest
+
+from turbogpt_amd.bridge import ModelConfig, Native
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {
+    "configs[3]": dict(d_model=768, depth=12, context=1024, batch=16, heads=12),
+    "configs[4]": dict(d_model=1024, depth=24, context=4096, batch=4, heads=16),
+}
+
+
+def weights(count, cfg, seed):
+    """N(0, 0.02) matrices, gamma = 1, beta = 0, in the flat order of include/tg_model.h."""
+    d, L, T, F = cfg["d_model"], cfg["depth"], cfg["context"], 4 * cfg["d_model"]
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal(count, dtype=np.float32) * 0.02).astype(np.float32)
+    at = 256 * d + T * d
+    for _ in range(L):
+        w[at:at + d], w[at + d:at + 2 * d] = 1.0, 0.0
+        at += 2 * d + 3 * d * d + d * d
+        w[at:at + d], w[at + d:at + 2 * d] = 1.0, 0.0
+        at += 2 * d + 2 * F * d
+    w[at:at + d], w[at + d:at + 2 * d] = 1.0, 0.0
+    assert at + 2 * d + 256 * d == count
+    return w
+
+
+def zipf_bytes(n, seed, s=1.1):
+    p = np.arange(1, 257, dtype=np.float64) ** -s
+    cdf = np.cumsum(p / p.sum())
+    return np.minimum(np.searchsorted(cdf, np.random.default_rng(seed).random(n)), 255).astype(np.uint8)
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_causality_and_gradient_identity_at_full_size(name):
+    cfg = CONFIGS[name]
+    B, T, d = cfg["batch"], cfg["context"], cfg["d_model"]
+    with Native(ModelConfig(**cfg)) as engine:
+        w = weights(engine.count, cfg, 3407)
+        engine.set_weights(w)
+        x = zipf_bytes(B * T, 71).reshape(B, T)
+        y = np.roll(x, -1, axis=1)
+        logits, grad, losses = engine.batch(x, y)
+        assert np.isfinite(logits).all() and np.isfinite(grad).all()
+        assert abs(float(losses.mean()) - np.log(256)) < 0.6  # ln 256 + half the logit variance
+        # the final LayerNorm output does not change when its input is scaled, so the loss does not depend
+        # on a common scale of (gamma_f, beta_f) only through the head: d loss / d log-scale of the head's
+        # input equals <grad_head, W_head> = <grad_gamma_f, gamma_f> + <grad_beta_f, beta_f>
+        head = slice(engine.count - 256 * d, engine.count)
+        lnf = slice(engine.count - 256 * d - 2 * d, engine.count - 256 * d)
+        lhs = float(np.dot(grad[head].astype(np.float64), w[head].astype(np.float64)))
+        rhs = float(np.dot(grad[lnf].astype(np.float64), w[lnf].astype(np.float64)))
+        assert abs(lhs - rhs) <= 2e-2 * max(abs(lhs), abs(rhs), 1e-3)
+        # causality, bit for bit: changing the last token of every sequence leaves every earlier position alone
+        x2 = x.copy()
+        x2[:, -1] ^= 0x55
+        logits2, _, _ = engine.batch(x2, y, backward=False)
+        a = logits.reshape(B, T, 256)[:, :-1]
+        b = logits2.reshape(B, T, 256)[:, :-1]
+        np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+        assert not np.array_equal(logits.reshape(B, T, 256)[:, -1], logits2.reshape(B, T, 256)[:, -1])
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_training_is_deterministic_and_learns_at_full_size(name):
+    cfg = CONFIGS[name]
+    steps = 6
+    data = zipf_bytes(1 << 22, 71)
+    runs = []
+    for _ in range(2):
+        with Native(ModelConfig(learning_rate=3e-4, beta1=0.9, beta2=0.95, weight_decay=0.1, clip=1.0, seed=3407,
+                                **cfg)) as engine:
+            engine.set_weights(weights(engine.count, cfg, 3407))
+            engine.set_data(data)
+            engine.train(steps)
+            runs.append(engine.training_losses(steps).copy())
+    np.testing.assert_array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32))
+    per_step = runs[0].mean(1)
+    assert np.isfinite(per_step).all()
+    assert abs(per_step[0] - np.log(256)) < 0.6
+    assert per_step[-1] < per_step[0] - 0.02  # six AdamW steps already lower the loss
