@@ -22,11 +22,13 @@ def test_library_exports_every_declared_symbol():
     lib = bridge.library()
     kernel = declared("tgk_kernels.h", "TGK_API")
     engine = declared("tg_runtime.h", "TG_API")
-    assert len(kernel) >= 18 and len(engine) >= 23
-    for name in kernel + engine:
+    checkpoint = declared("tg_checkpoint.h", "TG_API")
+    assert len(kernel) >= 18 and len(engine) >= 23 and len(checkpoint) == 3
+    for name in kernel + engine + checkpoint:
         assert hasattr(lib, name), name
     assert set(kernel) == set(bridge.KERNEL_ABI)
     assert set(engine) == set(bridge.ENGINE_ABI)
+    assert set(checkpoint) == set(bridge.CHECKPOINT_ABI)
 
 
 def test_pod_layouts_match_the_reference():

@@ -180,6 +180,31 @@ def test_one_launch_of_eight_steps_equals_eight_launches(orc, scheduled):
         b.close()
 
 
+def test_resume_from_a_checkpoint_file(orc, tmp_path):
+    """trainer.cpp:76-80 / checkpoint.cpp:506-579: weights and optimizer state written to a .pt file and
+    read into a fresh engine continue bit-identically to the uninterrupted run."""
+    from turbogpt_amd.bridge import read_checkpoint, write_checkpoint
+    cfg = ModelConfig(d_model=128, depth=2, context=128, batch=4)
+    data = orc.fill_zipf_bytes(8192, 4)
+    a, b = make_engine(orc, cfg, data), make_engine(orc, cfg, data)
+    try:
+        a.train(5)
+        m, v, step = a.optimizer_state()
+        path = tmp_path / "run.pt"
+        write_checkpoint(path, cfg, a.weights(), m, v, step, train_seconds=1.0)
+        state = read_checkpoint(path, expect=cfg)
+        assert state["step"] == 5
+        b.set_weights(state["weights"])
+        b.set_optimizer_state(state["momentum"], state["variance"], state["step"])
+        a.train(3)
+        b.train(3)
+        np.testing.assert_array_equal(a.training_losses(3), b.training_losses(3))
+        np.testing.assert_array_equal(a.weights().view(np.uint32), b.weights().view(np.uint32))
+    finally:
+        a.close()
+        b.close()
+
+
 def test_engine_error_paths(orc):
     cfg = ModelConfig(d_model=128, depth=1, context=128, batch=1)
     with Native(cfg) as engine:

@@ -107,6 +107,21 @@ ENGINE_ABI = {
     "tg_synchronize": (i32, [vp]),
     "tg_profile_step": (i32, [vp, vp, vp, i32]),
 }
+
+
+class Checkpoint(C.Structure):
+    """TgCheckpoint of include/tg_checkpoint.h."""
+    _fields_ = [("model", ModelConfig), ("parameter_count", i64), ("weights", vp), ("momentum", vp),
+                ("variance", vp), ("step", u64), ("scheduler", OneCycle), ("train_seconds", C.c_double),
+                ("final_loss_positions", i64), ("final_loss_sums", vp), ("final_loss_batches", u64)]
+
+
+# every symbol include/tg_checkpoint.h declares
+CHECKPOINT_ABI = {
+    "tg_checkpoint_write": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
+    "tg_checkpoint_inspect": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
+    "tg_checkpoint_read": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
+}
 CLASSES = ("gemm_fwd", "gemm_dgrad", "gemm_wgrad", "attn_fwd", "attn_bwd", "layernorm_fwd", "layernorm_bwd",
            "head", "other", "optimizer")
 
@@ -124,7 +139,7 @@ def library():
             raise RuntimeError(f"{path} is missing: build it with `python -m turbogpt_amd.build` "
                                "(there is no CPU or PyTorch fallback)")
         lib = C.CDLL(str(path))
-        for name, (restype, argtypes) in {**KERNEL_ABI, **ENGINE_ABI}.items():
+        for name, (restype, argtypes) in {**KERNEL_ABI, **ENGINE_ABI, **CHECKPOINT_ABI}.items():
             fn = getattr(lib, name)  # AttributeError if the symbol is not exported
             fn.restype, fn.argtypes = restype, argtypes
         _LIB = lib
@@ -235,3 +250,46 @@ class Native:
         logits = np.empty(self.config.vocab, np.float32)
         self.check(self.lib.tg_predict(self.handle, context.ctypes.data, logits.ctypes.data))
         return logits
+
+
+def write_checkpoint(path, model, weights, momentum, variance, step, scheduler=None, train_seconds=0.0,
+                     final_loss_sums=None, final_loss_batches=0):
+    """save_training_state of the reference (checkpoint.cpp:554-579) for the target model."""
+    import numpy as np
+    arrays = [np.ascontiguousarray(a, dtype=np.float32) for a in (weights, momentum, variance)]
+    sums = None if final_loss_sums is None else np.ascontiguousarray(final_loss_sums, dtype=np.float64)
+    c = Checkpoint()
+    c.model = model
+    c.parameter_count = arrays[0].size
+    c.weights, c.momentum, c.variance = (a.ctypes.data for a in arrays)
+    c.step = step
+    c.scheduler = scheduler if scheduler is not None else OneCycle(0)
+    c.train_seconds = train_seconds
+    c.final_loss_positions = 0 if sums is None else sums.size
+    c.final_loss_sums = None if sums is None else sums.ctypes.data
+    c.final_loss_batches = final_loss_batches
+    check(library().tg_checkpoint_write(os.fsencode(path), C.byref(c)))
+
+
+def read_checkpoint(path, expect=None):
+    """load_training_state (checkpoint.cpp:506-551): a dict of the file's contents; `expect`, a
+    ModelConfig, makes an architecture mismatch an error."""
+    import numpy as np
+    lib = library()
+    c = Checkpoint()
+    check(lib.tg_checkpoint_inspect(os.fsencode(path), C.byref(c)))
+    out = {name: np.empty(c.parameter_count, np.float32) for name in ("weights", "momentum", "variance")}
+    sums = np.empty(c.final_loss_positions, np.float64)
+    c.weights, c.momentum, c.variance = (out[n].ctypes.data for n in ("weights", "momentum", "variance"))
+    c.final_loss_sums = sums.ctypes.data if sums.size else None
+    if expect is not None:
+        c.model = expect
+    else:
+        c.model.d_model = 0
+    check(lib.tg_checkpoint_read(os.fsencode(path), C.byref(c)))
+    out.update(step=c.step, train_seconds=c.train_seconds, final_loss_sums=sums,
+               final_loss_batches=c.final_loss_batches,
+               scheduler={name: getattr(c.scheduler, name) for name, _ in OneCycle._fields_},
+               model={"depth": c.model.base.depth, "context": c.model.base.context, "d_model": c.model.d_model,
+                      "heads": c.model.heads, "vocab": c.model.vocab, "ffn": c.model.ffn})
+    return out
