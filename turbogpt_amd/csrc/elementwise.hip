@@ -118,9 +118,16 @@ __global__ __launch_bounds__(256) void embed_bwd_positions_kernel(const bf16_t *
 }
 
 // ---- LayerNorm --------------------------------------------------------------------------------
-// One wave per row, the row lives in registers (two-pass mean / variance).  NC = 16-byte chunks per
-// lane (D <= NC * 512): sizing the register tile to the row keeps occupancy up on narrow models.
-template <int NC>
+// A row lives in the registers of GROUP lanes (two-pass mean / variance), NC 16-byte chunks per lane
+// (D <= NC * GROUP * 8).  GROUP = 64: one row per wave.  GROUP = 32: two rows per wave, which fits
+// D = 768 (96 chunks = 32 x 3) without idle lane slots and keeps three loads per array in flight.
+template <int GROUP> TG_DEVICE float group_sum(float x) {
+#pragma unroll
+    for (int k = GROUP / 2; k; k >>= 1)
+        x += __shfl_xor(x, k, 64);
+    return x;
+}
+template <int NC, int GROUP>
 __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__restrict__ x,
                                                             const uint16_t *__restrict__ gamma_hi,
                                                             const uint16_t *__restrict__ gamma_lo,
@@ -128,36 +135,43 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
                                                             const uint16_t *__restrict__ beta_lo,
                                                             bf16_t *__restrict__ y, int rows, int D,
                                                             float eps) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, chunks = D >> 3;
+    constexpr int PER_BLOCK = 256 / GROUP; // rows a block works on at a time
+    const int lane = threadIdx.x & (GROUP - 1), slot = threadIdx.x / GROUP, chunks = D >> 3;
     const float inv_d = 1.0f / D;
-    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    // the row loop is uniform over the wave: a wave's second half may run one row past the end
+    for (int row0 = blockIdx.x * PER_BLOCK; row0 < rows; row0 += gridDim.x * PER_BLOCK) {
+        const int row = row0 + slot;
+        const bool live = row < rows;
         float v[NC][8];
         float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; ++j) {
-            const int c = lane + j * 64;
-            if (c < chunks) {
+            const int c = lane + j * GROUP;
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                v[j][k] = 0.f;
+            if (live && c < chunks) {
                 unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
                     sum += v[j][k];
             }
         }
-        const float mean = wave_sum(sum) * inv_d;
+        const float mean = group_sum<GROUP>(sum) * inv_d;
         float sq = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; ++j)
-            if (lane + j * 64 < chunks)
+            if (lane + j * GROUP < chunks)
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     v[j][k] -= mean;
                     sq += v[j][k] * v[j][k];
                 }
-        const float inv = 1.0f / sqrtf(wave_sum(sq) * inv_d + eps);
+        const float inv = 1.0f / sqrtf(group_sum<GROUP>(sq) * inv_d + eps);
 #pragma unroll
         for (int j = 0; j < NC; ++j) {
-            const int c = lane + j * 64;
-            if (c < chunks) {
+            const int c = lane + j * GROUP;
+            if (live && c < chunks) {
                 float gm[8], bt[8], o[8];
                 join8(gamma_hi + c * 8, gamma_lo + c * 8, gm);
                 join8(beta_hi + c * 8, beta_lo + c * 8, bt);
@@ -171,7 +185,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
 }
 
 // dx (+ residual), and per-block partial sums of dgamma / dbeta into partial[block][2][D].
-template <int NC>
+template <int NC, int GROUP>
 __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__restrict__ x,
                                                             const bf16_t *__restrict__ dy,
                                                             const uint16_t *__restrict__ gamma_hi,
@@ -179,26 +193,32 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
                                                             bf16_t *__restrict__ dx,
                                                             float *__restrict__ partial, int rows, int D,
                                                             float eps, int residual) {
-    extern __shared__ float lds[]; // [4 waves][2][D]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, chunks = D >> 3;
+    constexpr int PER_BLOCK = 256 / GROUP;
+    extern __shared__ float lds[]; // [PER_BLOCK row slots][2][D]
+    const int lane = threadIdx.x & (GROUP - 1), slot = threadIdx.x / GROUP, chunks = D >> 3;
     const float inv_d = 1.0f / D;
     float dg[NC][8], db[NC][8], gm[NC][8];
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-        const int c = lane + j * 64;
+        const int c = lane + j * GROUP;
 #pragma unroll
         for (int k = 0; k < 8; ++k)
             dg[j][k] = db[j][k] = gm[j][k] = 0.f;
         if (c < chunks)
             join8(gamma_hi + c * 8, gamma_lo + c * 8, gm[j]);
     }
-    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    for (int row0 = blockIdx.x * PER_BLOCK; row0 < rows; row0 += gridDim.x * PER_BLOCK) {
+        const int row = row0 + slot;
+        const bool live = row < rows;
         float v[NC][8], g[NC][8];
         float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; ++j) {
-            const int c = lane + j * 64;
-            if (c < chunks) {
+            const int c = lane + j * GROUP;
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                v[j][k] = g[j][k] = 0.f;
+            if (live && c < chunks) {
                 unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
                 unpack8(*reinterpret_cast<const u32x4 *>(dy + size_t(row) * D + c * 8), g[j]);
 #pragma unroll
@@ -206,21 +226,21 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
                     sum += v[j][k];
             }
         }
-        const float mean = wave_sum(sum) * inv_d;
+        const float mean = group_sum<GROUP>(sum) * inv_d;
         float sq = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; ++j)
-            if (lane + j * 64 < chunks)
+            if (lane + j * GROUP < chunks)
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     v[j][k] -= mean;
                     sq += v[j][k] * v[j][k];
                 }
-        const float inv = 1.0f / sqrtf(wave_sum(sq) * inv_d + eps);
+        const float inv = 1.0f / sqrtf(group_sum<GROUP>(sq) * inv_d + eps);
         float s1 = 0.f, s2 = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; ++j)
-            if (lane + j * 64 < chunks)
+            if (live && lane + j * GROUP < chunks)
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     const float z = v[j][k] * inv, dz = g[j][k] * gm[j][k];
@@ -230,12 +250,12 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
                     dg[j][k] += g[j][k] * z;
                     db[j][k] += g[j][k];
                 }
-        s1 = wave_sum(s1) * inv_d;
-        s2 = wave_sum(s2) * inv_d;
+        s1 = group_sum<GROUP>(s1) * inv_d;
+        s2 = group_sum<GROUP>(s2) * inv_d;
 #pragma unroll
         for (int j = 0; j < NC; ++j) {
-            const int c = lane + j * 64;
-            if (c < chunks) {
+            const int c = lane + j * GROUP;
+            if (live && c < chunks) {
                 float o[8];
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
@@ -253,10 +273,10 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
             }
         }
     }
-    float *mine = lds + wave * 2 * D;
+    float *mine = lds + slot * 2 * D;
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-        const int c = lane + j * 64;
+        const int c = lane + j * GROUP;
         if (c < chunks)
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
@@ -265,9 +285,13 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
             }
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < 2 * D; i += 256)
-        partial[size_t(blockIdx.x) * 2 * D + i] =
-            (lds[i] + lds[2 * D + i]) + (lds[4 * D + i] + lds[6 * D + i]);
+    for (int i = threadIdx.x; i < 2 * D; i += 256) {
+        float sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < PER_BLOCK; ++r) // fixed order
+            sum += lds[r * 2 * D + i];
+        partial[size_t(blockIdx.x) * 2 * D + i] = sum;
+    }
 }
 // dgamma[c] (+)= sum_b partial[b][0][c], dbeta likewise.  16 columns x 16 row phases per block; every
 // thread keeps 8 independent loads in flight; phases are combined in a fixed order.
@@ -582,6 +606,16 @@ extern "C" int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab,
     });
 }
 
+// lanes per row and 16-byte chunks per lane: half a wave per row where that leaves fewer idle lane slots
+struct LayerNormShape {
+    int group, chunks;
+};
+static LayerNormShape layernorm_shape(int D) {
+    const int chunks = D / 8, per64 = (chunks + 63) / 64, per32 = (chunks + 31) / 32;
+    if (per32 < 2 * per64 && per32 <= 3)
+        return {32, per32}; // 1 or 3 chunks per lane (2 never wins over a whole wave)
+    return {64, per64 <= 2 ? per64 : 4};
+}
 extern "C" int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint16_t *x,
                                  const uint16_t *gamma_hi, const uint16_t *gamma_lo,
                                  const uint16_t *beta_hi, const uint16_t *beta_lo, uint16_t *y, float eps) {
@@ -594,16 +628,22 @@ extern "C" int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint
         aligned(gamma_lo, "layernorm: gamma_lo");
         aligned(beta_hi, "layernorm: beta_hi");
         aligned(beta_lo, "layernorm: beta_lo");
-        const dim3 grid(grid_for(rows, 4, 8192));
-        if (D <= 512)
-            hipLaunchKernelGGL(layernorm_fwd_kernel<1>, grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo, beta_hi,
-                               beta_lo, y, rows, D, eps);
-        else if (D <= 1024)
-            hipLaunchKernelGGL(layernorm_fwd_kernel<2>, grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo, beta_hi,
-                               beta_lo, y, rows, D, eps);
+        const LayerNormShape shape = layernorm_shape(D);
+        const dim3 grid(grid_for(rows, 256 / shape.group, 8192));
+#define TG_LN_FWD(NC, GROUP)                                                                                      \
+    hipLaunchKernelGGL((layernorm_fwd_kernel<NC, GROUP>), grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo,      \
+                       beta_hi, beta_lo, y, rows, D, eps)
+        if (shape.group == 32 && shape.chunks == 1)
+            TG_LN_FWD(1, 32);
+        else if (shape.group == 32)
+            TG_LN_FWD(3, 32);
+        else if (shape.chunks == 1)
+            TG_LN_FWD(1, 64);
+        else if (shape.chunks == 2)
+            TG_LN_FWD(2, 64);
         else
-            hipLaunchKernelGGL(layernorm_fwd_kernel<4>, grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo, beta_hi,
-                               beta_lo, y, rows, D, eps);
+            TG_LN_FWD(4, 64);
+#undef TG_LN_FWD
         check_hip(hipGetLastError(), "layernorm_fwd launch: ");
     });
 }
@@ -631,16 +671,20 @@ extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint
                 "layernorm_bwd: workspace too small (see tgk_layernorm_bwd_workspace)");
         const int blocks = layernorm_bwd_blocks(rows);
         float *partial = static_cast<float *>(workspace);
-        const size_t lds = size_t(8) * D * sizeof(float);
-        if (D <= 512)
-            hipLaunchKernelGGL(layernorm_bwd_kernel<1>, dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,
-                               gamma_lo, dx, partial, rows, D, eps, residual);
-        else if (D <= 1024)
-            hipLaunchKernelGGL(layernorm_bwd_kernel<2>, dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,
-                               gamma_lo, dx, partial, rows, D, eps, residual);
+        // one row per wave here: two rows per wave cost registers (148 for D = 768) and LDS that lower the
+        // occupancy, and measured slower
+        const int per_lane = (D / 8 + 63) / 64;
+        const size_t lds = size_t(4) * 2 * D * sizeof(float);
+#define TG_LN_BWD(NC, GROUP)                                                                                      \
+    hipLaunchKernelGGL((layernorm_bwd_kernel<NC, GROUP>), dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,  \
+                       gamma_lo, dx, partial, rows, D, eps, residual)
+        if (per_lane == 1)
+            TG_LN_BWD(1, 64);
+        else if (per_lane == 2)
+            TG_LN_BWD(2, 64);
         else
-            hipLaunchKernelGGL(layernorm_bwd_kernel<4>, dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,
-                               gamma_lo, dx, partial, rows, D, eps, residual);
+            TG_LN_BWD(4, 64);
+#undef TG_LN_BWD
         hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3(2 * D / 16), dim3(256), 0, stream, partial, blocks, D,
                            dgamma, dbeta, accumulate);
         check_hip(hipGetLastError(), "layernorm_bwd launch: ");
