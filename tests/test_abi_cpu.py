@@ -93,3 +93,19 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setenv("TURBOGPT_LIBRARY", str(tmp_path / "absent.so"))
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         bridge.library()
+
+
+def test_headers_are_plain_c_and_the_host_program_links(tmp_path):
+    """The boundary is a C ABI: every header under include/ compiles as C99 (-pedantic) and as C++17 on its
+    own, and the host program (turbogpt_amd/host/train_bytes.cpp) builds with plain g++ against the
+    library and refuses to run without arguments."""
+    import subprocess
+    from turbogpt_amd import build as native
+    for header in sorted((ROOT / "include").glob("*.h")):
+        for compiler, std, lang in (("gcc", "-std=c99", "c"), ("g++", "-std=c++17", "c++")):
+            done = subprocess.run([compiler, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", lang,
+                                   str(header)], capture_output=True, text=True)
+            assert done.returncode == 0, f"{header.name} as {lang}: {done.stderr}"
+    program = native.build_host()
+    done = subprocess.run([str(program)], capture_output=True, text=True)
+    assert done.returncode == 1 and "usage: train_bytes --data FILE" in done.stderr

@@ -205,6 +205,39 @@ def test_resume_from_a_checkpoint_file(orc, tmp_path):
         b.close()
 
 
+def test_host_program_trains_and_resumes(orc, tmp_path):
+    """turbogpt_amd/host/train_bytes (plain g++ over the C ABI): the loss falls; 12 steps in one run equal
+    6 steps + checkpoint + 6 resumed steps, to the last printed digit (trainer.cpp:51-80,105-121)."""
+    import json
+    import subprocess
+    from turbogpt_amd import build as native
+    program = native.HOST_PROGRAM
+    assert program.exists(), "build it with python -m turbogpt_amd.build"
+    data = tmp_path / "bytes.bin"
+    data.write_bytes(orc.fill_zipf_bytes(1 << 16, 4).tobytes())
+    common = [str(program), "--data", str(data), "--depth", "2", "--context", "128", "--batch", "4", "--d_model", "128",
+              "--chunk", "3", "--tokens", str(12 * 4 * 128)]
+
+    def run(*extra):
+        done = subprocess.run(common + list(extra), capture_output=True, text=True, timeout=120)
+        assert done.returncode == 0, done.stderr
+        return [json.loads(line) for line in done.stdout.splitlines()]
+
+    whole = run("--save", str(tmp_path / "whole.pt"))
+    assert [r["step"] for r in whole[:-1]] == [3, 6, 9, 12] and whole[-1]["steps"] == 12
+    assert whole[-2]["loss"] < whole[0]["loss"] - 0.05 and len(whole[-1]["sample"]) == 68
+    # a run cut after six steps: same schedule (--tokens), fewer steps trained
+    first = subprocess.run(common + ["--save", str(tmp_path / "half.pt"), "--chunk", "6"], capture_output=True, text=True,
+                           timeout=120, env={"TRAIN_BYTES_STOP_AFTER": "6", **__import__("os").environ})
+    assert first.returncode == 0, first.stderr
+    resumed = run("--load", str(tmp_path / "half.pt"), "--save", str(tmp_path / "resumed.pt"))
+    assert resumed[-1]["steps"] == 12 and resumed[-1]["final_loss"] == whole[-1]["final_loss"]
+    from turbogpt_amd.bridge import read_checkpoint
+    a, b = read_checkpoint(tmp_path / "whole.pt"), read_checkpoint(tmp_path / "resumed.pt")
+    np.testing.assert_array_equal(a["weights"].view(np.uint32), b["weights"].view(np.uint32))
+    assert a["step"] == b["step"] == 12
+
+
 def test_engine_error_paths(orc):
     cfg = ModelConfig(d_model=128, depth=1, context=128, batch=1)
     with Native(cfg) as engine:

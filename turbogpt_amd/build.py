@@ -13,6 +13,8 @@ HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 OBJ = CSRC / "_obj"
 LIBRARY = HERE / "libturbogpt.so"
+HOST_SOURCE = HERE / "host" / "train_bytes.cpp"
+HOST_PROGRAM = HERE / "host" / "train_bytes"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -47,12 +49,24 @@ def _compile(source, force):
     return obj
 
 
+def build_host():
+    """The host program over the C ABI (host/train_bytes.cpp), with plain g++ against the library."""
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-Wextra", "-I", str(HERE.parent / "include"),
+           str(HOST_SOURCE), "-L", str(HERE), "-lturbogpt", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath-link,/opt/rocm/lib",
+           "-o", str(HOST_PROGRAM)]
+    result = subprocess.run(cmd, capture_output=True, text=True)
+    if result.returncode:
+        raise RuntimeError(f"g++ failed on {HOST_SOURCE.name}:\n{result.stderr}")
+    return HOST_PROGRAM
+
+
 def build(force=False, jobs=8):
     OBJ.mkdir(exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objects = list(pool.map(lambda s: _compile(s, force), _sources()))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIBRARY), *map(str, objects)]
     subprocess.run(cmd, check=True)
+    build_host()
     return LIBRARY
 
 
