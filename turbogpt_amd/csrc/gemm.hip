@@ -21,6 +21,7 @@
 // fp32 stores and a fused epilogue on the fragment.  Fragments of the next k-step are read while
 // the current MFMAs run, also across the per-k-tile barrier.
 #include "common.h"
+#include <atomic>
 #include "../../include/tgk_kernels.h"
 
 namespace {
@@ -410,16 +411,26 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
 }
 
 // ---- host dispatch -------------------------------------------------------------------------
+// Per-device facts are cached per device: several engines may run on different GPUs of one process.
+constexpr int MAX_DEVICES = 64;
+int current_device() {
+    int device = 0;
+    check_hip(hipGetDevice(&device));
+    if (device < 0 || device >= MAX_DEVICES)
+        throw std::runtime_error("gemm: device index out of range");
+    return device;
+}
 int compute_units() {
-    static int cached = 0;
-    if (!cached) {
-        int device = 0;
+    static std::atomic<int> cached[MAX_DEVICES];
+    const int device = current_device();
+    int units = cached[device].load(std::memory_order_relaxed);
+    if (!units) {
         hipDeviceProp_t prop{};
-        check_hip(hipGetDevice(&device));
         check_hip(hipGetDeviceProperties(&prop, device));
-        cached = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        units = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        cached[device].store(units, std::memory_order_relaxed);
     }
-    return cached;
+    return units;
 }
 
 enum Tile { TILE_NONE, TILE_128x128, TILE_128x192 };
@@ -469,12 +480,13 @@ void launch_gemm(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, 
                  int K, int splits, int max_blocks, const Epilogue &epilogue) {
     auto kernel = gemm_kernel<BM, BN, S, AKC, BKC, Epilogue>;
     constexpr size_t lds = lds_bytes<BM, BN, S, Epilogue>();
-    static bool configured = false;
-    if (!configured) {
+    static std::atomic<bool> configured[MAX_DEVICES]; // the LDS opt-in is a per-device attribute of the kernel
+    const int device = current_device();
+    if (!configured[device].load(std::memory_order_acquire)) {
         check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)),
                   "gemm LDS size: ");
-        configured = true;
+        configured[device].store(true, std::memory_order_release);
     }
     const int tiles_m = M / BM, tiles_n = N / BN, tiles = tiles_m * tiles_n, items = tiles * splits;
     const int blocks = items < max_blocks ? items : max_blocks;
