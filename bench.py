@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Headline benchmark: training tokens/sec of the byte-level GPT d768 L12 H12 T1024 B16
-(BASELINE.json configs[3]) on one MI355X, through the tg_* C ABI.
+(the fourth benchmark configuration, configs[3]) on one MI355X, through the tg_* C ABI.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--kernels]
 
@@ -27,7 +27,7 @@ M = B * T
 # mean over the four projection shapes of 2 * (M*K + N*K + M*N) bytes: operands read and the result written once
 ALGORITHMIC_BYTES_PER_LAUNCH = sum(2 * (M * k + n * k + M * n) for n, k in
                                    [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
-# HBM bytes per launch of that kernel measured with rocprofv3 counters (profiles/gemm_kc_ks_hbm_traffic.md)
+# HBM bytes per launch of that kernel, measured with rocprofv3 FETCH_SIZE / WRITE_SIZE runs of --traffic-probe
 HBM_TRAFFIC_PER_LAUNCH = 150.5e6
 
 
@@ -287,8 +287,8 @@ def main():
                                "dgrads: QKV, attention-out, MLP-up, MLP-down)",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": HBM_TRAFFIC_PER_LAUNCH,
-                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated; "
-                                     "profiles/gemm_kc_ks_hbm_traffic.md)",
+                     "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE of --traffic-probe, "
+                                     "calibrated on a copy of known size)",
                      "algorithmic_bytes_per_launch": ALGORITHMIC_BYTES_PER_LAUNCH,
                      "flops_per_launch": flops_per_launch, "avg_launch_ms": round(launch_ms, 5)},
         "classes": classes,
