@@ -56,8 +56,9 @@ typedef struct StepRates {
 typedef struct Engine Engine;
 
 TG_API const char *tg_error(void);                                   /* runtime.h:14 */
-/* runtime.h:15.  The reference builds its width-16 network from this struct alone; that
- * architecture is not part of this library, so tg_create reports an error naming tg_create_ex. */
+/* runtime.h:15, cuda/runtime.cu:62-155: the reference's own width-16 network (RMSNorm, partial RoPE,
+ * arg-max attention, SwiGLU; AdamW + Muon), with the reference's limits: depth 4/8, context 4/8, batch >= 4,
+ * batch*context divisible by 16, ns_steps 1..10, inflight 1.  Flat weight order: model.h:12-37. */
 TG_API Engine *tg_create(const Config *config);
 /* Validates the shape, allocates every device buffer once (weights hi/lo, m, v, gradient, saved
  * activations, workspaces, loss history); NULL on failure (cuda/runtime.cu:62-155). */

@@ -133,8 +133,8 @@ TGK_API int tgk_sumsq_partials(hipStream_t stream, const float *g, size_t n, flo
  * from the folded partials when clip > 0, m += (1-b1)(g-m), v = b2 v + (1-b2) g^2,
  * w = w (1 - lr*wd) - (lr/bc1) m / (sqrt(v)/sqrt(bc2) + eps), bias corrections from `step`
  * (0-based) with the current beta1.  segment_starts (device, sorted, first = 0) and
- * segment_flags (device, bit 0 = apply weight decay) describe the decay groups
- * (cuda/optim.cuh:5-15).  n and all segment starts multiples of 4. */
+ * segment_flags (device, bit 0 = apply weight decay, bit 1 = leave the segment untouched: it belongs
+ * to another optimizer) describe the parameter groups (cuda/optim.cuh:5-15).  n and all segment starts multiples of 4. */
 TGK_API int tgk_adamw(hipStream_t stream, size_t n, uint16_t *weight_hi, uint16_t *weight_lo, float *m,
                       float *v, const float *g, const float *norm_partials, int norm_count,
                       const int64_t *segment_starts, const uint8_t *segment_flags, int segments, float lr,
@@ -147,6 +147,32 @@ TGK_API int tgk_sample_batch(hipStream_t stream, const uint8_t *data, int64_t si
 /* out[p] = mean over the batch of token_loss[b*context + p], in double (cuda/trainer.cuh:79-100). */
 TGK_API int tgk_position_means(hipStream_t stream, const float *token_loss, int batch, int context,
                                float *out);
+
+/* ---- The reference's own width-16 network (config.h:4, model.h:12-37): RMSNorm, partial RoPE, causal
+ * arg-max attention with a GELU gate, SwiGLU(48), 4 heads of 4, vocabulary 256.  These four calls stand in
+ * for forward / backward / optimize of the persistent kernel (cuda/model.cuh:8-99, cuda/optim.cuh:17-119)
+ * when an engine is created from the plain Config.  depth 1..8, context 1..8 (the RoPE table of
+ * cuda/attention.cuh:7-14 has eight entries); weights in the flat order of model.h:12-37. ---- */
+TGK_API int tgk_w16_parameter_count(int depth);
+/* bytes of device workspace (256-byte aligned) that forward fills and backward consumes */
+TGK_API size_t tgk_w16_workspace(int depth, int batch, int context);
+/* x, y: [batch*context] tokens and targets.  token_losses[batch*context]; logits (may be NULL) receives
+ * [batch*context][256] floats; with_gradient != 0 also leaves RN_bf16((softmax - onehot) / tokens) in the
+ * workspace for tgk_w16_backward (cuda/model.cuh:54-55). */
+TGK_API int tgk_w16_forward(hipStream_t stream, int depth, int batch, int context, const uint16_t *weight_hi,
+                            const uint16_t *weight_lo, const uint8_t *x, const uint8_t *y, void *workspace,
+                            float *token_losses, float *logits, int with_gradient);
+/* after tgk_w16_forward(with_gradient) on the same workspace: every element of gradient[parameter_count]
+ * is overwritten; weight gradients are folded in a fixed order (no atomics). */
+TGK_API int tgk_w16_backward(hipStream_t stream, int depth, int batch, int context, const uint16_t *weight_hi,
+                             const uint16_t *weight_lo, const uint8_t *x, void *workspace, float *gradient);
+/* Muon update of the 5*depth hidden matrices (cuda/optim.cuh:17-62, :107-118): Nesterov momentum, bf16
+ * Newton-Schulz with the 3.4445 / -4.775 / 2.0315 quintic, decoupled decay, lr * sqrt(max(1, rows/cols)).
+ * The clip scale is folded from the same norm partials tgk_adamw uses; the other parameters are
+ * tgk_adamw's, whose segment flag bit 1 makes it leave the hidden matrices alone. */
+TGK_API int tgk_w16_muon(hipStream_t stream, int depth, uint16_t *weight_hi, uint16_t *weight_lo, float *momentum,
+                         const float *gradient, const float *norm_partials, int norm_count, float clip, float lr,
+                         float momentum_rate, float weight_decay, int ns_steps);
 
 #ifdef __cplusplus
 }

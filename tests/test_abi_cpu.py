@@ -65,8 +65,14 @@ def test_onecycle_point_known_answers_and_checker(orc):
 
 def test_create_rejects_bad_configurations_before_touching_a_device():
     lib = bridge.library()
-    assert lib.tg_create(C.byref(bridge.Config())) is None
-    assert b"tg_create_ex" in lib.tg_error()
+    # the plain Config builds the reference's width-16 network, with the reference's limits (cuda/runtime.cu:65-78)
+    for kwargs, needle in [(dict(batch=16, context=5), b"depth 4/8, context 4/8"), (dict(batch=16, depth=3), b"depth 4/8"),
+                           (dict(batch=2), b"batch at least 4"), (dict(batch=6), b"divisible by 16"),
+                           (dict(batch=16, inflight=0), b"inflight must be 1..256"),
+                           (dict(batch=16, inflight=2), b"inflight"), (dict(batch=16, ns_steps=0), b"ns_steps")]:
+        assert lib.tg_create(C.byref(bridge.Config(**kwargs))) is None
+        assert needle in lib.tg_error(), (kwargs, lib.tg_error())
+    assert lib.tg_create(None) is None
     cases = [(dict(d_model=100), b"d_model"), (dict(d_model=256, heads=3), b"head_dim"),
              (dict(d_model=256, vocab=100), b"vocabulary"), (dict(d_model=256, depth=0), b"depth"),
              (dict(d_model=256, depth=2, context=100), b"context"),
@@ -86,6 +92,8 @@ def test_kernel_entry_points_validate_arguments_on_the_host():
     assert lib.tgk_gemm_wgrad_workspace(64, 100, 128) == 0
     assert lib.tgk_attn_bwd_workspace(2, 3, 128) == 2 * (2 * 3 * 128 * 4)
     assert lib.tgk_layernorm_bwd_workspace(16384, 768) == 1024 * 2 * 768 * 4
+    assert lib.tgk_w16_parameter_count(4) == 21648 and lib.tgk_w16_parameter_count(8) == 35088  # model.h:12-37
+    assert lib.tgk_w16_workspace(4, 16, 8) % 256 == 0 and lib.tgk_w16_workspace(4, 16, 9) == 0
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -38,6 +38,11 @@ KERNEL_ABI = {
                         C.c_uint64]),
     "tgk_sample_batch": (i32, [vp, vp, i64, C.c_uint64, C.c_uint64, i32, i32, vp, vp]),
     "tgk_position_means": (i32, [vp, vp, i32, i32, vp]),
+    "tgk_w16_parameter_count": (i32, [i32]),
+    "tgk_w16_workspace": (C.c_size_t, [i32, i32, i32]),
+    "tgk_w16_forward": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, i32]),
+    "tgk_w16_backward": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, vp]),
+    "tgk_w16_muon": (i32, [vp, i32, vp, vp, vp, vp, vp, i32, f32, f32, f32, f32, i32]),
 }
 u64 = C.c_uint64
 
@@ -153,14 +158,18 @@ def check(status):
 
 
 class Native:
-    """One engine, as in tests/bridge.py:29-81 of the reference, over tg_create_ex."""
+    """One engine, as in tests/bridge.py:29-81 of the reference: tg_create for a plain Config (the reference's
+    width-16 network), tg_create_ex for a ModelConfig."""
 
     def __init__(self, config):
         import numpy as np
         self.np = np
         self.config = config
         self.lib = library()
-        self.handle = self.lib.tg_create_ex(C.byref(config))
+        self.base = config if isinstance(config, Config) else config.base
+        self.vocab = 256 if isinstance(config, Config) else config.vocab
+        create = self.lib.tg_create if isinstance(config, Config) else self.lib.tg_create_ex
+        self.handle = create(C.byref(config))
         if not self.handle:
             raise RuntimeError(self.lib.tg_error().decode())
         self.count = self.lib.tg_parameter_count(self.handle)
@@ -212,7 +221,7 @@ class Native:
         self.check(self.lib.tg_train(self.handle, steps))
 
     def training_losses(self, count):
-        out = self.np.empty((count, self.config.base.context), self.np.float32)
+        out = self.np.empty((count, self.base.context), self.np.float32)
         self.check(self.lib.tg_get_training_losses(self.handle, out.ctypes.data, count))
         return out
 
@@ -233,10 +242,10 @@ class Native:
 
     def batch(self, x, y, backward=True):
         np = self.np
-        base = self.config.base
+        base = self.base
         x, y = np.ascontiguousarray(x, dtype=np.uint8), np.ascontiguousarray(y, dtype=np.uint8)
         assert x.shape == y.shape == (base.batch, base.context)
-        logits = np.empty((*x.shape, self.config.vocab), np.float32)
+        logits = np.empty((*x.shape, self.vocab), np.float32)
         grad = np.empty(self.count, np.float32) if backward else None
         losses = np.empty(base.context, np.float32)
         self.check(self.lib.tg_batch(self.handle, x.ctypes.data, y.ctypes.data, logits.ctypes.data,
@@ -246,8 +255,8 @@ class Native:
     def predict(self, context):
         np = self.np
         context = np.ascontiguousarray(context, dtype=np.uint8)
-        assert context.size == self.config.base.context
-        logits = np.empty(self.config.vocab, np.float32)
+        assert context.size == self.base.context
+        logits = np.empty(self.vocab, np.float32)
         self.check(self.lib.tg_predict(self.handle, context.ctypes.data, logits.ctypes.data))
         return logits
 

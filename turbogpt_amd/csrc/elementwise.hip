@@ -397,7 +397,7 @@ struct AdamArgs {
     float lr, beta1, beta2, eps, weight_decay, bc1, sqrt_bc2, clip;
 };
 // cuda/optim.cuh:67-106 on the (hi bf16, lo u16) weight halves (cuda/ops.cuh:6-14).
-// bounds: sorted starts of `segments` parameter ranges, bit 0 of flags[s] = weight decay.
+// bounds: sorted starts of `segments` parameter ranges, bit 0 of flags[s] = weight decay, bit 1 = skip.
 __global__ __launch_bounds__(256) void adamw_kernel(bf16_t *__restrict__ hi, uint16_t *__restrict__ lo,
                                                     float *__restrict__ m, float *__restrict__ v,
                                                     const float *__restrict__ g, size_t n,
@@ -433,6 +433,8 @@ __global__ __launch_bounds__(256) void adamw_kernel(bf16_t *__restrict__ hi, uin
             else
                 hi_s = mid - 1;
         }
+        if (flags[lo_s] & 2) // owned by another optimizer (Muon, cuda/optim.cuh:94-96)
+            continue;
         const float decay = (flags[lo_s] & 1) ? a.weight_decay : 0.f;
         const f32x4 gv = *reinterpret_cast<const f32x4 *>(g + i);
         f32x4 mv = *reinterpret_cast<const f32x4 *>(m + i), vv = *reinterpret_cast<const f32x4 *>(v + i);

@@ -64,6 +64,7 @@ struct Engine {
     std::vector<void *> allocations;
     size_t allocated_bytes = 0;
     int compute_units = 0;
+    bool width16 = false; // the reference's own network, created from the plain Config
 
     uint16_t *weight_hi = nullptr, *weight_lo = nullptr;
     uint16_t *weight_t = nullptr; // every matrix of weight_hi transposed ([In][Out]), same offsets
@@ -162,12 +163,19 @@ struct Engine {
     const uint16_t *wt(int64_t offset) const { return weight_t + offset; }
     // forward projections read the transposed weights: call after every change of weight_hi
     void refresh_transposed() {
+        if (width16)
+            return;
         ok(tgk_transpose_batch(stream, weight_hi, weight_t, transpose_jobs, transpose_count, transpose_tiles));
     }
 
     // cuda/model.cuh:8-59.  evaluate: logits stay logits; otherwise they are replaced by dlogits.
     void forward(const uint8_t *tokens_in, const uint8_t *targets, bool with_gradient, float *logits_out) {
         const Config &c = config.base;
+        if (width16) {
+            OP(TG_CLASS_OTHER, tgk_w16_forward(stream, c.depth, c.batch, c.context, weight_hi, weight_lo, tokens_in,
+                                               targets, workspace, token_losses, logits_out, with_gradient ? 1 : 0));
+            return;
+        }
         const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
         OP(TG_CLASS_OTHER, tgk_embed_fwd(stream, M, T, d, tokens_in, w(layout.embedding), w(layout.positions), x[0]));
@@ -195,6 +203,11 @@ struct Engine {
     // cuda/model.cuh:61-99.  Every element of `gradient` is overwritten: nothing needs zeroing.
     void backward(const uint8_t *tokens_in) {
         const Config &c = config.base;
+        if (width16) {
+            OP(TG_CLASS_OTHER, tgk_w16_backward(stream, c.depth, c.batch, c.context, weight_hi, weight_lo, tokens_in,
+                                                workspace, gradient));
+            return;
+        }
         const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
         float *g = gradient;
@@ -229,16 +242,22 @@ struct Engine {
     // cuda/optim.cuh:66-106 for optimizer step `at` (0-based)
     void optimize(uint64_t at) {
         const Config &c = config.base;
-        float lr = c.learning_rate, beta1 = c.beta1;
-        if (!schedule.empty()) {
+        float lr = c.learning_rate, beta1 = c.beta1, muon_lr = c.muon_lr, muon_momentum = c.momentum;
+        if (!schedule.empty()) { // cuda/optim.cuh:81-88: one point drives both learning rates and both momenta
             lr *= schedule[at].multiplier;
-            beta1 = schedule[at].momentum;
+            muon_lr *= schedule[at].multiplier;
+            beta1 = muon_momentum = schedule[at].momentum;
         }
         if (c.clip > 0)
             OP(TG_CLASS_OPTIMIZER, tgk_sumsq_partials(stream, gradient, size_t(layout.count), norm_partials, NormPartials));
         OP(TG_CLASS_OPTIMIZER, tgk_adamw(stream, size_t(layout.count), weight_hi, weight_lo, momentum, variance, gradient,
                      norm_partials, NormPartials, segment_starts, segment_flags, segments, lr, beta1, c.beta2,
                      c.epsilon, c.weight_decay, c.clip, at));
+        if (width16) { // the hidden matrices, which the AdamW segments skip (cuda/optim.cuh:107-118)
+            OP(TG_CLASS_OPTIMIZER, tgk_w16_muon(stream, c.depth, weight_hi, weight_lo, momentum, gradient, norm_partials,
+                                                NormPartials, c.clip, muon_lr, muon_momentum, c.weight_decay, c.ns_steps));
+            return;
+        }
         OP(TG_CLASS_OPTIMIZER, tgk_transpose_batch(stream, weight_hi, weight_t, transpose_jobs, transpose_count,
                                                    transpose_tiles));
     }
@@ -351,10 +370,91 @@ void build_segments(Engine *e) {
 
 } // namespace
 
-TG_API Engine *tg_create(const Config *) {
-    tg_last_error = "tg_create builds the reference's fixed width-16 network, which this library does not "
-                    "contain; describe the model with TgModelConfig and call tg_create_ex";
-    return nullptr;
+// cuda/runtime.cu:62-155: the reference's own width-16 network (config.h:4)
+TG_API Engine *tg_create(const Config *c) {
+    Engine *e = nullptr;
+    try {
+        if (!c)
+            throw std::runtime_error("Missing configuration");
+        if ((c->context != 4 && c->context != 8) || (c->depth != 4 && c->depth != 8) || c->batch < 4 ||
+            c->batch * c->context % 16)
+            throw std::runtime_error("Supported: depth 4/8, context 4/8, batch at least 4 with "
+                                     "batch*context divisible by 16");
+        if (c->inflight < 1 || c->inflight > 256)
+            throw std::runtime_error("inflight must be 1..256");
+        if (c->inflight > 1)
+            throw std::runtime_error("inflight > 1 (stale-gradient overlap) is not built; use inflight = 1");
+        if (c->ns_steps < 1 || c->ns_steps > 10)
+            throw std::runtime_error("ns_steps must be 1..10");
+        int devices = 0;
+        check_hip(hipGetDeviceCount(&devices), "device query: ");
+        if (c->device < 0 || c->device >= devices)
+            throw std::runtime_error("No such device");
+        check_hip(hipSetDevice(c->device));
+        hipDeviceProp_t prop{};
+        check_hip(hipGetDeviceProperties(&prop, c->device));
+        if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            throw std::runtime_error(std::string("Requires an MI355X-class device (gfx950), found ") +
+                                     prop.gcnArchName);
+        e = new Engine;
+        e->width16 = true;
+        e->config.base = *c;
+        e->config.d_model = 16, e->config.heads = 4, e->config.vocab = 256, e->config.ffn = 48;
+        e->config.ln_eps = 1e-6f;
+        e->layout.count = tgk_w16_parameter_count(c->depth);
+        e->compute_units = prop.multiProcessorCount;
+        check_hip(hipStreamCreate(&e->stream));
+        const size_t P = size_t(e->layout.count), M = size_t(e->tokens());
+        e->allocate(e->weight_hi, P);
+        e->allocate(e->weight_lo, P);
+        e->allocate(e->momentum, P);
+        e->allocate(e->variance, P);
+        e->allocate(e->gradient, P);
+        e->allocate(e->norm_partials, NormPartials);
+        e->allocate(e->token_losses, M);
+        e->allocate(e->loss_history, size_t(MaxLaunchSteps) * c->context);
+        e->allocate(e->input, M);
+        e->allocate(e->target, M);
+        // AdamW owns the embedding, the RMSNorm scales and the head (decayed); Muon the hidden matrices
+        // (cuda/optim.cuh:5-15).  Flat order per layer (model.h:20-31): scale 16, qkv 768, attention 256, scale 16,
+        // gate 768, up 768, down 768.
+        std::vector<int64_t> starts;
+        std::vector<uint8_t> flags;
+        int64_t at = 0;
+        const auto add = [&](int64_t size, uint8_t flag) {
+            if (flags.empty() || flags.back() != flag) {
+                starts.push_back(at);
+                flags.push_back(flag);
+            }
+            at += size;
+        };
+        add(256 * 16, 0);
+        for (int l = 0; l < c->depth; ++l) {
+            add(16, 0);
+            add(48 * 16 + 16 * 16, 2);
+            add(16, 0);
+            add(3 * 48 * 16, 2);
+        }
+        add(16, 0);
+        add(256 * 16, 1);
+        if (at != int64_t(P))
+            throw std::runtime_error("internal: width-16 segment table does not cover the parameters");
+        e->segments = int(starts.size());
+        e->allocate(e->segment_starts, starts.size(), false);
+        e->allocate(e->segment_flags, flags.size(), false);
+        e->upload(e->segment_starts, starts.data(), starts.size());
+        e->upload(e->segment_flags, flags.data(), flags.size());
+        e->workspace_bytes = tgk_w16_workspace(c->depth, c->batch, c->context);
+        uint8_t *ws = nullptr;
+        e->allocate(ws, e->workspace_bytes, false);
+        e->workspace = ws;
+        e->sync();
+        return e;
+    } catch (const std::exception &error) {
+        tg_last_error = error.what();
+        delete e;
+        return nullptr;
+    }
 }
 
 TG_API Engine *tg_create_ex(const TgModelConfig *model) {
