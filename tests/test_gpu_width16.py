@@ -190,7 +190,7 @@ def test_stream_evaluation(context):
         engine.set_data(data)
         for _ in range(3):
             loss = engine.batch(x, y, False)[2]
-            np.testing.assert_allclose(loss, expected, rtol=1e-3, atol=1e-3)
+            np.testing.assert_allclose(loss, expected, rtol=1e-6, atol=1e-6)
 
 
 def test_training_follows_the_checker(orc):
