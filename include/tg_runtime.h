@@ -29,7 +29,7 @@ typedef struct Config {
     float beta1, beta2, momentum;
     float weight_decay, epsilon, clip;
     uint64_t seed;
-    int inflight; /* only 1 (synchronous) is built */
+    int inflight; /* 1: synchronous; 2..16: that many batches in flight on versioned, stale weights */
 } Config;
 
 /* The model shape the reference has no room for.  Byte-level GPT: pre-LayerNorm blocks,
@@ -58,7 +58,7 @@ typedef struct Engine Engine;
 TG_API const char *tg_error(void);                                   /* runtime.h:14 */
 /* runtime.h:15, cuda/runtime.cu:62-155: the reference's own width-16 network (RMSNorm, partial RoPE,
  * arg-max attention, SwiGLU; AdamW + Muon), with the reference's limits: depth 4/8, context 4/8, batch >= 4,
- * batch*context divisible by 16, ns_steps 1..10, inflight 1.  Flat weight order: model.h:12-37. */
+ * batch*context divisible by 16, ns_steps 1..10, inflight 1..16.  Flat weight order: model.h:12-37. */
 TG_API Engine *tg_create(const Config *config);
 /* Validates the shape, allocates every device buffer once (weights hi/lo, m, v, gradient, saved
  * activations, workspaces, loss history); NULL on failure (cuda/runtime.cu:62-155). */

@@ -68,15 +68,17 @@ def test_create_rejects_bad_configurations_before_touching_a_device():
     # the plain Config builds the reference's width-16 network, with the reference's limits (cuda/runtime.cu:65-78)
     for kwargs, needle in [(dict(batch=16, context=5), b"depth 4/8, context 4/8"), (dict(batch=16, depth=3), b"depth 4/8"),
                            (dict(batch=2), b"batch at least 4"), (dict(batch=6), b"divisible by 16"),
-                           (dict(batch=16, inflight=0), b"inflight must be 1..256"),
-                           (dict(batch=16, inflight=2), b"inflight"), (dict(batch=16, ns_steps=0), b"ns_steps")]:
+                           (dict(batch=16, inflight=0), b"inflight must be 1..16"),
+                           (dict(batch=16, inflight=17), b"inflight must be 1..16"),
+                           (dict(batch=16, inflight=2, blocks=4), b"synchronous training only"),
+                           (dict(batch=16, ns_steps=0), b"ns_steps")]:
         assert lib.tg_create(C.byref(bridge.Config(**kwargs))) is None
         assert needle in lib.tg_error(), (kwargs, lib.tg_error())
     assert lib.tg_create(None) is None
     cases = [(dict(d_model=100), b"d_model"), (dict(d_model=256, heads=3), b"head_dim"),
              (dict(d_model=256, vocab=100), b"vocabulary"), (dict(d_model=256, depth=0), b"depth"),
              (dict(d_model=256, depth=2, context=100), b"context"),
-             (dict(d_model=256, depth=2, context=128, inflight=2), b"inflight"),
+             (dict(d_model=256, depth=2, context=128, inflight=17), b"inflight must be 1..16"),
              (dict(d_model=256, depth=2, context=128, batch=0), b"batch"),
              (dict(d_model=256, ffn=1000, depth=2, context=128), b"ffn")]
     for kwargs, needle in cases:

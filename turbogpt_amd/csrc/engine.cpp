@@ -16,6 +16,7 @@ namespace {
 
 constexpr int MaxLaunchSteps = 4096; // cuda/types.cuh:10
 constexpr int NormPartials = 1024;
+constexpr int MaxInFlight = 16; // batches in flight, each with its own stream and saved activations
 
 struct LayerBuffers {
     bf16_t *n1, *qkv, *o, *mid, *n2, *u, *a;
@@ -57,6 +58,27 @@ StepRates onecycle_point(const OneCycle &s, int step) {
 
 } // namespace
 
+// Everything one batch in flight owns: its stream, its tokens, its saved activations and its gradient.
+// A synchronous engine has one slot on the engine's stream; inflight = K gives K slots on K streams
+// (the worker teams of cuda/pipeline.cuh:52-92).
+struct Slot {
+    hipStream_t stream = nullptr;
+    hipEvent_t ready = nullptr; // the gradient of the slot's latest step is complete
+    uint8_t *input = nullptr, *target = nullptr;
+    float *token_losses = nullptr, *gradient = nullptr;
+    std::vector<bf16_t *> x; // x[l] = input of block l; x[depth] = output of the last block
+    std::vector<LayerBuffers> layers;
+    bf16_t *nf = nullptr, *logits = nullptr, *dh = nullptr, *t1 = nullptr, *du = nullptr, *dqkv = nullptr;
+    void *workspace = nullptr;
+};
+// One immutable copy of the weights: a batch reads a single version from its first kernel to its last
+// (cuda/pipeline.cuh:36-38).  inflight = K keeps K + 1 of them in a ring; a synchronous engine one.
+struct Version {
+    uint16_t *hi = nullptr, *lo = nullptr;
+    uint16_t *t = nullptr;     // every matrix of hi transposed ([In][Out]), same offsets (wide model only)
+    hipEvent_t done = nullptr; // the optimizer step that wrote this version has finished
+};
+
 struct Engine {
     TgModelConfig config{};
     TgParameterLayout layout{};
@@ -66,28 +88,27 @@ struct Engine {
     int compute_units = 0;
     bool width16 = false; // the reference's own network, created from the plain Config
 
-    uint16_t *weight_hi = nullptr, *weight_lo = nullptr;
-    uint16_t *weight_t = nullptr; // every matrix of weight_hi transposed ([In][Out]), same offsets
+    std::vector<Slot> slots;
+    std::vector<Version> versions;
     void *transpose_jobs = nullptr;
     int transpose_count = 0, transpose_tiles = 0;
-    float *momentum = nullptr, *variance = nullptr, *gradient = nullptr;
-    float *norm_partials = nullptr, *token_losses = nullptr, *loss_history = nullptr;
+    float *momentum = nullptr, *variance = nullptr;
+    float *norm_partials = nullptr, *loss_history = nullptr;
     int64_t *segment_starts = nullptr;
     uint8_t *segment_flags = nullptr;
     int segments = 0;
-    uint8_t *data = nullptr, *input = nullptr, *target = nullptr;
+    uint8_t *data = nullptr;
     int64_t data_size = 0;
-
-    std::vector<bf16_t *> x; // x[l] = input of block l; x[depth] = output of the last block
-    std::vector<LayerBuffers> layers;
-    bf16_t *nf = nullptr, *logits = nullptr, *dh = nullptr, *t1 = nullptr, *du = nullptr, *dqkv = nullptr;
     float *logits_f32 = nullptr;
-    void *workspace = nullptr;
     size_t workspace_bytes = 0;
 
     std::vector<StepRates> schedule;
     uint64_t step = 0;
+    uint64_t floor = 0; // oldest weight version that exists: the step at the last tg_set_weights / _set_optimizer_state
     int last_train_steps = 0;
+    std::vector<int> version_trace; // weight version each step of the last tg_train read
+    uint64_t total_staleness = 0;
+    int max_staleness = 0;
 
     // optional per-class timing of one step (tg_profile_step): event pairs around every launch
     struct Span {
@@ -110,7 +131,7 @@ struct Engine {
     struct Scope {
         Engine *e;
         size_t index = 0;
-        Scope(Engine *engine, int cls) : e(engine) {
+        Scope(Engine *engine, int cls) : e(engine) { // profiling exists for synchronous engines: one stream
             if (!e->profiling)
                 return;
             index = e->spans.size();
@@ -135,7 +156,13 @@ struct Engine {
             check_hip(hipMemsetAsync(raw, 0, n * sizeof(T), stream));
     }
     void use_device() const { check_hip(hipSetDevice(config.base.device)); }
-    void sync() const { check_hip(hipStreamSynchronize(stream)); }
+    void sync() const { // every stream: the engine is quiescent afterwards
+        for (const Slot &slot : slots)
+            if (slot.stream && slot.stream != stream)
+                check_hip(hipStreamSynchronize(slot.stream));
+        check_hip(hipStreamSynchronize(stream));
+    }
+    Version &current() { return versions[step % versions.size()]; }
     template <class T> void upload(T *device, const T *host, size_t n) {
         check_hip(hipMemcpyAsync(device, host, n * sizeof(T), hipMemcpyHostToDevice, stream));
     }
@@ -144,10 +171,22 @@ struct Engine {
     }
     ~Engine() { // cuda/engine_internal.h:28-37
         (void)hipSetDevice(config.base.device);
+        for (Slot &slot : slots)
+            if (slot.stream && slot.stream != stream)
+                (void)hipStreamSynchronize(slot.stream);
         if (stream)
             (void)hipStreamSynchronize(stream);
         for (void *allocation : allocations)
             (void)hipFree(allocation);
+        for (Slot &slot : slots) {
+            if (slot.ready)
+                (void)hipEventDestroy(slot.ready);
+            if (slot.stream && slot.stream != stream)
+                (void)hipStreamDestroy(slot.stream);
+        }
+        for (Version &version : versions)
+            if (version.done)
+                (void)hipEventDestroy(version.done);
         for (Span &span : spans) {
             (void)hipEventDestroy(span.start);
             (void)hipEventDestroy(span.stop);
@@ -158,24 +197,31 @@ struct Engine {
             (void)hipStreamDestroy(stream);
     }
 
-    const uint16_t *w(int64_t offset) const { return weight_hi + offset; }
-    const uint16_t *wl(int64_t offset) const { return weight_lo + offset; }
-    const uint16_t *wt(int64_t offset) const { return weight_t + offset; }
-    // forward projections read the transposed weights: call after every change of weight_hi
-    void refresh_transposed() {
+    // forward projections read the transposed weights: call after every change of a version's hi half
+    void refresh_transposed(const Version &v) {
         if (width16)
             return;
-        ok(tgk_transpose_batch(stream, weight_hi, weight_t, transpose_jobs, transpose_count, transpose_tiles));
+        ok(tgk_transpose_batch(stream, v.hi, v.t, transpose_jobs, transpose_count, transpose_tiles));
     }
 
     // cuda/model.cuh:8-59.  evaluate: logits stay logits; otherwise they are replaced by dlogits.
-    void forward(const uint8_t *tokens_in, const uint8_t *targets, bool with_gradient, float *logits_out) {
+    // On the slot's stream, with one weight version, from the slot's tokens.
+    void forward(Slot &s, const Version &v, bool with_gradient, float *logits_out) {
         const Config &c = config.base;
+        hipStream_t stream = s.stream;
+        const uint8_t *tokens_in = s.input, *targets = s.target;
+        float *token_losses = s.token_losses;
         if (width16) {
-            OP(TG_CLASS_OTHER, tgk_w16_forward(stream, c.depth, c.batch, c.context, weight_hi, weight_lo, tokens_in,
-                                               targets, workspace, token_losses, logits_out, with_gradient ? 1 : 0));
+            OP(TG_CLASS_OTHER, tgk_w16_forward(stream, c.depth, c.batch, c.context, v.hi, v.lo, tokens_in, targets,
+                                               s.workspace, token_losses, logits_out, with_gradient ? 1 : 0));
             return;
         }
+        const auto w = [&](int64_t offset) { return v.hi + offset; };
+        const auto wl = [&](int64_t offset) { return v.lo + offset; };
+        const auto wt = [&](int64_t offset) { return v.t + offset; };
+        std::vector<bf16_t *> &x = s.x;
+        std::vector<LayerBuffers> &layers = s.layers;
+        bf16_t *nf = s.nf, *logits = s.logits;
         const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
         OP(TG_CLASS_OTHER, tgk_embed_fwd(stream, M, T, d, tokens_in, w(layout.embedding), w(layout.positions), x[0]));
@@ -201,13 +247,22 @@ struct Engine {
     }
 
     // cuda/model.cuh:61-99.  Every element of `gradient` is overwritten: nothing needs zeroing.
-    void backward(const uint8_t *tokens_in) {
+    void backward(Slot &s, const Version &v) {
         const Config &c = config.base;
+        hipStream_t stream = s.stream;
+        const uint8_t *tokens_in = s.input;
+        float *gradient = s.gradient;
+        void *workspace = s.workspace;
         if (width16) {
-            OP(TG_CLASS_OTHER, tgk_w16_backward(stream, c.depth, c.batch, c.context, weight_hi, weight_lo, tokens_in,
-                                                workspace, gradient));
+            OP(TG_CLASS_OTHER, tgk_w16_backward(stream, c.depth, c.batch, c.context, v.hi, v.lo, tokens_in, workspace,
+                                                gradient));
             return;
         }
+        const auto w = [&](int64_t offset) { return v.hi + offset; };
+        const auto wl = [&](int64_t offset) { return v.lo + offset; };
+        std::vector<bf16_t *> &x = s.x;
+        std::vector<LayerBuffers> &layers = s.layers;
+        bf16_t *nf = s.nf, *logits = s.logits, *dh = s.dh, *t1 = s.t1, *du = s.du, *dqkv = s.dqkv;
         const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
         float *g = gradient;
@@ -239,9 +294,11 @@ struct Engine {
                                          workspace, workspace_bytes));
     }
 
-    // cuda/optim.cuh:66-106 for optimizer step `at` (0-based)
-    void optimize(uint64_t at) {
+    // cuda/optim.cuh:66-106 for optimizer step `at` (0-based), on the engine's stream: gradient -> the weights of
+    // version `to` (which already hold the previous version's values)
+    void optimize(uint64_t at, const float *gradient, Version &to) {
         const Config &c = config.base;
+        uint16_t *weight_hi = to.hi, *weight_lo = to.lo, *weight_t = to.t;
         float lr = c.learning_rate, beta1 = c.beta1, muon_lr = c.muon_lr, muon_momentum = c.momentum;
         if (!schedule.empty()) { // cuda/optim.cuh:81-88: one point drives both learning rates and both momenta
             lr *= schedule[at].multiplier;
@@ -261,20 +318,50 @@ struct Engine {
         OP(TG_CLASS_OPTIMIZER, tgk_transpose_batch(stream, weight_hi, weight_t, transpose_jobs, transpose_count,
                                                    transpose_tiles));
     }
-    // one full training step; shared by tg_train and tg_profile_step
-    void train_step(uint64_t at, float *history_row) {
+    // batch `at`: sample, forward, loss row, backward, on one slot with one weight version
+    void batch_gradient(Slot &s, const Version &v, uint64_t at, float *history_row) {
         const Config &c = config.base;
-        OP(TG_CLASS_OTHER, tgk_sample_batch(stream, data, data_size, c.seed, at, c.batch, c.context, input, target));
-        forward(input, target, true, nullptr);
-        OP(TG_CLASS_OTHER, tgk_position_means(stream, token_losses, c.batch, c.context, history_row));
-        backward(input);
-        optimize(at);
+        hipStream_t stream = s.stream;
+        OP(TG_CLASS_OTHER, tgk_sample_batch(stream, data, data_size, c.seed, at, c.batch, c.context, s.input, s.target));
+        forward(s, v, true, nullptr);
+        OP(TG_CLASS_OTHER, tgk_position_means(stream, s.token_losses, c.batch, c.context, history_row));
+        backward(s, v);
+    }
+    // One training step.  Synchronous engine: everything in order on the one stream, weights updated in place
+    // (cuda/trainer.cuh:109-124).  inflight = K (cuda/pipeline.cuh:40-126 as streams and events): batch `at`
+    // runs on slot at % K with the oldest version the ring still guarantees, max(floor, at - K + 1), so it
+    // only waits for optimizer step at - K (which also freed the slot's gradient); the optimizer step waits for
+    // the batch, copies version `at` into ring place at + 1 and updates it there.  The choice is made on the
+    // host, so a run is reproducible; the staleness bound at - K + 1 <= version <= at is the reference's.
+    void train_step(uint64_t at, float *history_row, int *trace) {
+        const uint64_t K = slots.size(), ring = versions.size();
+        if (K == 1) {
+            batch_gradient(slots[0], versions[0], at, history_row);
+            optimize(at, slots[0].gradient, versions[0]);
+            *trace = int(at);
+            return;
+        }
+        Slot &s = slots[at % K];
+        const uint64_t read = std::max(floor, at + 1 >= K ? at + 1 - K : 0);
+        check_hip(hipStreamWaitEvent(s.stream, versions[read % ring].done, 0));
+        batch_gradient(s, versions[read % ring], at, history_row);
+        check_hip(hipEventRecord(s.ready, s.stream));
+        Version &from = versions[at % ring], &to = versions[(at + 1) % ring];
+        check_hip(hipStreamWaitEvent(stream, s.ready, 0));
+        const size_t bytes = size_t(layout.count) * 2;
+        check_hip(hipMemcpyAsync(to.hi, from.hi, bytes, hipMemcpyDeviceToDevice, stream));
+        check_hip(hipMemcpyAsync(to.lo, from.lo, bytes, hipMemcpyDeviceToDevice, stream));
+        optimize(at, s.gradient, to);
+        check_hip(hipEventRecord(to.done, stream));
+        *trace = int(read);
+        total_staleness += at - read;
+        max_staleness = std::max(max_staleness, int(at - read));
     }
 
     void read_losses(float *out) { // cuda/runtime.cu:279-290
         const Config &c = config.base;
         std::vector<float> losses(static_cast<size_t>(tokens()));
-        download(losses.data(), token_losses, losses.size());
+        download(losses.data(), slots[0].token_losses, losses.size());
         sync();
         for (int p = 0; p < c.context; ++p) {
             double sum = 0;
@@ -303,10 +390,37 @@ void validate(const TgModelConfig &m) {
         throw std::runtime_error("Supported: context a multiple of 128");
     if (c.batch < 1 || int64_t(c.batch) * c.context > (int64_t(1) << 24))
         throw std::runtime_error("Supported: batch >= 1 with batch*context <= 2^24 tokens");
-    if (c.inflight != 1)
-        throw std::runtime_error("inflight must be 1: the stale-gradient pipeline is not built");
+    if (c.inflight < 1 || c.inflight > MaxInFlight)
+        throw std::runtime_error("inflight must be 1.." + std::to_string(MaxInFlight));
     if (!(m.ln_eps > 0))
         throw std::runtime_error("ln_eps must be positive");
+}
+
+// Streams, events and the buffers every model kind needs per slot and per weight version.
+void build_slots(Engine *e, int inflight, bool transposed_copies) {
+    const size_t P = size_t(e->layout.count), M = size_t(e->tokens());
+    e->slots.resize(size_t(inflight));
+    e->versions.resize(inflight > 1 ? size_t(inflight) + 1 : 1);
+    for (Slot &slot : e->slots) {
+        if (inflight > 1) {
+            check_hip(hipStreamCreate(&slot.stream)); // default priority
+            check_hip(hipEventCreateWithFlags(&slot.ready, hipEventDisableTiming));
+        } else {
+            slot.stream = e->stream;
+        }
+        e->allocate(slot.input, M);
+        e->allocate(slot.target, M);
+        e->allocate(slot.token_losses, M);
+        e->allocate(slot.gradient, P);
+    }
+    for (Version &version : e->versions) {
+        e->allocate(version.hi, P);
+        e->allocate(version.lo, P);
+        if (transposed_copies)
+            e->allocate(version.t, P);
+        if (inflight > 1)
+            check_hip(hipEventCreateWithFlags(&version.done, hipEventDisableTiming));
+    }
 }
 
 void build_transpose_jobs(Engine *e) {
@@ -380,10 +494,10 @@ TG_API Engine *tg_create(const Config *c) {
             c->batch * c->context % 16)
             throw std::runtime_error("Supported: depth 4/8, context 4/8, batch at least 4 with "
                                      "batch*context divisible by 16");
-        if (c->inflight < 1 || c->inflight > 256)
-            throw std::runtime_error("inflight must be 1..256");
-        if (c->inflight > 1)
-            throw std::runtime_error("inflight > 1 (stale-gradient overlap) is not built; use inflight = 1");
+        if (c->inflight < 1 || c->inflight > MaxInFlight)
+            throw std::runtime_error("inflight must be 1.." + std::to_string(MaxInFlight));
+        if (c->inflight > 1 && c->blocks)
+            throw std::runtime_error("model.blocks applies to synchronous training only");
         if (c->ns_steps < 1 || c->ns_steps > 10)
             throw std::runtime_error("ns_steps must be 1..10");
         int devices = 0;
@@ -404,17 +518,12 @@ TG_API Engine *tg_create(const Config *c) {
         e->layout.count = tgk_w16_parameter_count(c->depth);
         e->compute_units = prop.multiProcessorCount;
         check_hip(hipStreamCreate(&e->stream));
-        const size_t P = size_t(e->layout.count), M = size_t(e->tokens());
-        e->allocate(e->weight_hi, P);
-        e->allocate(e->weight_lo, P);
+        const size_t P = size_t(e->layout.count);
+        build_slots(e, c->inflight, false);
         e->allocate(e->momentum, P);
         e->allocate(e->variance, P);
-        e->allocate(e->gradient, P);
         e->allocate(e->norm_partials, NormPartials);
-        e->allocate(e->token_losses, M);
         e->allocate(e->loss_history, size_t(MaxLaunchSteps) * c->context);
-        e->allocate(e->input, M);
-        e->allocate(e->target, M);
         // AdamW owns the embedding, the RMSNorm scales and the head (decayed); Muon the hidden matrices
         // (cuda/optim.cuh:5-15).  Flat order per layer (model.h:20-31): scale 16, qkv 768, attention 256, scale 16,
         // gate 768, up 768, down 768.
@@ -445,9 +554,11 @@ TG_API Engine *tg_create(const Config *c) {
         e->upload(e->segment_starts, starts.data(), starts.size());
         e->upload(e->segment_flags, flags.data(), flags.size());
         e->workspace_bytes = tgk_w16_workspace(c->depth, c->batch, c->context);
-        uint8_t *ws = nullptr;
-        e->allocate(ws, e->workspace_bytes, false);
-        e->workspace = ws;
+        for (Slot &slot : e->slots) {
+            uint8_t *ws = nullptr;
+            e->allocate(ws, e->workspace_bytes, false);
+            slot.workspace = ws;
+        }
         e->sync();
         return e;
     } catch (const std::exception &error) {
@@ -484,40 +595,36 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
         const Config &c = model->base;
         const size_t P = size_t(e->layout.count), M = size_t(e->tokens()), d = size_t(model->d_model);
         const size_t F = size_t(model->ffn), V = size_t(model->vocab);
-        e->allocate(e->weight_hi, P);
-        e->allocate(e->weight_lo, P);
-        e->allocate(e->weight_t, P);
+        build_slots(e, c.inflight, true);
         e->allocate(e->momentum, P);
         e->allocate(e->variance, P);
-        e->allocate(e->gradient, P);
         e->allocate(e->norm_partials, NormPartials);
-        e->allocate(e->token_losses, M);
         e->allocate(e->loss_history, size_t(MaxLaunchSteps) * c.context);
-        e->allocate(e->input, M);
-        e->allocate(e->target, M);
         build_segments(e);
         build_transpose_jobs(e);
-        e->x.resize(c.depth + 1);
-        e->layers.resize(c.depth);
-        for (int l = 0; l <= c.depth; ++l)
-            e->allocate(e->x[l], M * d, false);
-        for (int l = 0; l < c.depth; ++l) {
-            LayerBuffers &b = e->layers[l];
-            e->allocate(b.n1, M * d, false);
-            e->allocate(b.qkv, M * 3 * d, false);
-            e->allocate(b.o, M * d, false);
-            e->allocate(b.lse, size_t(c.batch) * model->heads * c.context, false);
-            e->allocate(b.mid, M * d, false);
-            e->allocate(b.n2, M * d, false);
-            e->allocate(b.u, M * F, false);
-            e->allocate(b.a, M * F, false);
+        for (Slot &slot : e->slots) {
+            slot.x.resize(c.depth + 1);
+            slot.layers.resize(c.depth);
+            for (int l = 0; l <= c.depth; ++l)
+                e->allocate(slot.x[l], M * d, false);
+            for (int l = 0; l < c.depth; ++l) {
+                LayerBuffers &b = slot.layers[l];
+                e->allocate(b.n1, M * d, false);
+                e->allocate(b.qkv, M * 3 * d, false);
+                e->allocate(b.o, M * d, false);
+                e->allocate(b.lse, size_t(c.batch) * model->heads * c.context, false);
+                e->allocate(b.mid, M * d, false);
+                e->allocate(b.n2, M * d, false);
+                e->allocate(b.u, M * F, false);
+                e->allocate(b.a, M * F, false);
+            }
+            e->allocate(slot.nf, M * d, false);
+            e->allocate(slot.logits, M * V, false);
+            e->allocate(slot.dh, M * d, false);
+            e->allocate(slot.t1, M * d, false);
+            e->allocate(slot.du, M * F, false);
+            e->allocate(slot.dqkv, M * 3 * d, false);
         }
-        e->allocate(e->nf, M * d, false);
-        e->allocate(e->logits, M * V, false);
-        e->allocate(e->dh, M * d, false);
-        e->allocate(e->t1, M * d, false);
-        e->allocate(e->du, M * F, false);
-        e->allocate(e->dqkv, M * 3 * d, false);
         size_t need = tgk_attn_bwd_workspace(c.batch, model->heads, c.context);
         need = std::max(need, tgk_layernorm_bwd_workspace(int(M), int(d)));
         need = std::max(need, tgk_embed_bwd_workspace(int(M), int(d)));
@@ -527,9 +634,11 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(d), int(d)));
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(3 * d), int(d)));
         e->workspace_bytes = need;
-        uint8_t *ws = nullptr;
-        e->allocate(ws, need, false);
-        e->workspace = ws;
+        for (Slot &slot : e->slots) {
+            uint8_t *ws = nullptr;
+            e->allocate(ws, need, false);
+            slot.workspace = ws;
+        }
         e->sync();
         return e;
     } catch (const std::exception &error) {
@@ -579,12 +688,16 @@ TG_API int tg_set_weights(Engine *e, const float *weights) {
             high[i] = uint16_t(bits >> 16);
             low[i] = uint16_t(bits);
         }
-        e->upload(e->weight_hi, high.data(), n);
-        e->upload(e->weight_lo, low.data(), n);
+        e->sync(); // nothing may still read the version that is overwritten
+        e->step = 0;
+        e->floor = 0;
+        e->total_staleness = 0, e->max_staleness = 0;
+        Version &v = e->current();
+        e->upload(v.hi, high.data(), n);
+        e->upload(v.lo, low.data(), n);
         check_hip(hipMemsetAsync(e->momentum, 0, n * 4, e->stream));
         check_hip(hipMemsetAsync(e->variance, 0, n * 4, e->stream));
-        e->refresh_transposed();
-        e->step = 0;
+        e->refresh_transposed(v);
         e->sync();
     });
 }
@@ -596,8 +709,9 @@ TG_API int tg_get_weights(Engine *e, float *weights) {
         e->use_device();
         const size_t n = size_t(e->layout.count);
         std::vector<uint16_t> high(n), low(n);
-        e->download(high.data(), e->weight_hi, n);
-        e->download(low.data(), e->weight_lo, n);
+        e->sync();
+        e->download(high.data(), e->current().hi, n);
+        e->download(low.data(), e->current().lo, n);
         e->sync();
         for (size_t i = 0; i < n; ++i) {
             const uint32_t bits = (uint32_t(high[i]) << 16) | low[i];
@@ -610,6 +724,7 @@ TG_API int tg_get_optimizer_state(Engine *e, float *momentum, float *variance, u
         if (!momentum || !variance || !step)
             throw std::runtime_error("Missing optimizer state output");
         e->use_device();
+        e->sync();
         e->download(momentum, e->momentum, size_t(e->layout.count));
         e->download(variance, e->variance, size_t(e->layout.count));
         e->sync();
@@ -621,9 +736,21 @@ TG_API int tg_set_optimizer_state(Engine *e, const float *momentum, const float 
         if (!momentum || !variance)
             throw std::runtime_error("Missing optimizer state input");
         e->use_device();
+        e->sync();
+        // the weights keep their values but become version `step`: move them to that place of the ring
+        Version &from = e->current();
+        Version &to = e->versions[step % e->versions.size()];
+        if (&from != &to) {
+            const size_t bytes = size_t(e->layout.count) * 2;
+            check_hip(hipMemcpyAsync(to.hi, from.hi, bytes, hipMemcpyDeviceToDevice, e->stream));
+            check_hip(hipMemcpyAsync(to.lo, from.lo, bytes, hipMemcpyDeviceToDevice, e->stream));
+            if (to.t)
+                check_hip(hipMemcpyAsync(to.t, from.t, bytes, hipMemcpyDeviceToDevice, e->stream));
+        }
         e->upload(e->momentum, momentum, size_t(e->layout.count));
         e->upload(e->variance, variance, size_t(e->layout.count));
         e->step = step;
+        e->floor = step;
         e->sync();
     });
 }
@@ -677,8 +804,10 @@ TG_API int tg_train(Engine *e, int steps) {
         if (!e->schedule.empty() && e->step + uint64_t(steps) > e->schedule.size())
             throw std::runtime_error("Training would exceed the OneCycle schedule");
         e->use_device();
+        e->version_trace.assign(size_t(steps), 0);
         for (int i = 0; i < steps; ++i)
-            e->train_step(e->step + uint64_t(i), e->loss_history + size_t(i) * e->config.base.context);
+            e->train_step(e->step + uint64_t(i), e->loss_history + size_t(i) * e->config.base.context,
+                          &e->version_trace[size_t(i)]);
         e->last_train_steps = steps;
         e->step += uint64_t(steps);
     });
@@ -691,25 +820,28 @@ TG_API int tg_get_training_losses(Engine *e, float *losses, int count) {
         if (count < 0 || count > e->last_train_steps)
             throw std::runtime_error("Training loss count exceeds the last launch");
         e->use_device();
+        e->sync(); // the rows are written on the slots' streams
         e->download(losses, e->loss_history, size_t(count) * e->config.base.context);
         e->sync();
     });
 }
-// cuda/runtime.cu:243-262: synchronous engines train step s on weight version s
+// cuda/runtime.cu:243-262: the weight version each step of the last tg_train read (a synchronous engine
+// trains step s on version s)
 TG_API int tg_training_versions(Engine *e, int *out, int count) {
     return guarded([&] {
         if (count < 0 || count > e->last_train_steps || (!out && count))
             throw std::runtime_error("Version trace exceeds last training launch");
         for (int i = 0; i < count; ++i)
-            out[i] = int(e->step) - e->last_train_steps + i;
+            out[i] = e->version_trace[size_t(i)];
     });
 }
-TG_API int tg_pipeline_stats(Engine *, double *mean, int *maximum) {
+// cuda/runtime.cu:263-278
+TG_API int tg_pipeline_stats(Engine *e, double *mean, int *maximum) {
     return guarded([&] {
         if (!mean || !maximum)
             throw std::runtime_error("Missing pipeline statistics output");
-        *mean = 0;
-        *maximum = 0;
+        *mean = e->step ? double(e->total_staleness) / double(e->step) : 0;
+        *maximum = e->max_staleness;
     });
 }
 
@@ -723,14 +855,17 @@ TG_API int tg_batch(Engine *e, const uint8_t *x, const uint8_t *y, float *logits
         const size_t M = size_t(e->tokens()), V = size_t(e->config.vocab);
         if (!e->logits_f32)
             e->allocate(e->logits_f32, M * V, false);
-        e->upload(e->input, x, M);
-        e->upload(e->target, y, M);
-        e->forward(e->input, e->target, gradient != nullptr, e->logits_f32);
+        e->sync(); // fixed batches run on slot 0 with the newest weights, after everything in flight
+        Slot &slot = e->slots[0];
+        check_hip(hipMemcpyAsync(slot.input, x, M, hipMemcpyHostToDevice, slot.stream));
+        check_hip(hipMemcpyAsync(slot.target, y, M, hipMemcpyHostToDevice, slot.stream));
+        e->forward(slot, e->current(), gradient != nullptr, e->logits_f32);
         if (gradient)
-            e->backward(e->input);
+            e->backward(slot, e->current());
+        check_hip(hipStreamSynchronize(slot.stream));
         e->download(logits, e->logits_f32, M * V);
         if (gradient)
-            e->download(gradient, e->gradient, size_t(e->layout.count));
+            e->download(gradient, slot.gradient, size_t(e->layout.count));
         e->read_losses(loss);
     });
 }
@@ -747,9 +882,12 @@ TG_API int tg_predict(Engine *e, const uint8_t *context, float *logits) {
         std::vector<uint8_t> input(M), target(M, 0);
         for (int b = 0; b < c.batch; ++b)
             std::copy(context, context + c.context, input.begin() + size_t(b) * c.context);
-        e->upload(e->input, input.data(), M);
-        e->upload(e->target, target.data(), M);
-        e->forward(e->input, e->target, false, e->logits_f32);
+        e->sync();
+        Slot &slot = e->slots[0];
+        check_hip(hipMemcpyAsync(slot.input, input.data(), M, hipMemcpyHostToDevice, slot.stream));
+        check_hip(hipMemcpyAsync(slot.target, target.data(), M, hipMemcpyHostToDevice, slot.stream));
+        e->forward(slot, e->current(), false, e->logits_f32);
+        check_hip(hipStreamSynchronize(slot.stream));
         e->download(logits, e->logits_f32 + size_t(c.context - 1) * V, V);
         e->sync();
     });
@@ -759,14 +897,16 @@ TG_API int tg_optimizer_test(Engine *e, const float *gradient, int steps) {
     return guarded([&] {
         if (!gradient)
             throw std::runtime_error("Missing gradient");
+        if (e->slots.size() > 1)
+            throw std::runtime_error("Optimizer oracle requires synchronous configuration");
         if (steps < 1 || steps > 64)
             throw std::runtime_error("steps must be 1..64");
         if (!e->schedule.empty() && e->step + uint64_t(steps) > e->schedule.size())
             throw std::runtime_error("Optimizer test would exceed the OneCycle schedule");
         e->use_device();
-        e->upload(e->gradient, gradient, size_t(e->layout.count));
+        e->upload(e->slots[0].gradient, gradient, size_t(e->layout.count));
         for (int i = 0; i < steps; ++i)
-            e->optimize(e->step + uint64_t(i));
+            e->optimize(e->step + uint64_t(i), e->slots[0].gradient, e->versions[0]);
         e->step += uint64_t(steps);
         e->sync();
     });
@@ -781,12 +921,15 @@ TG_API int tg_profile_step(Engine *e, float *class_ms, int *class_launches, int 
             throw std::runtime_error("tg_profile_step needs room for TG_CLASSES entries");
         if (!e->data)
             throw std::runtime_error("Load data first");
+        if (e->slots.size() > 1)
+            throw std::runtime_error("tg_profile_step requires synchronous configuration (inflight 1)");
         if (!e->schedule.empty() && e->step + 1 > e->schedule.size())
             throw std::runtime_error("Training would exceed the OneCycle schedule");
         e->use_device();
+        e->version_trace.assign(1, 0);
         e->profiling = true;
         try {
-            e->train_step(e->step, e->loss_history);
+            e->train_step(e->step, e->loss_history, e->version_trace.data());
         } catch (...) {
             e->profiling = false;
             throw;
