@@ -23,9 +23,11 @@ def test_library_exports_every_declared_symbol():
     kernel = declared("tgk_kernels.h", "TGK_API")
     engine = declared("tg_runtime.h", "TG_API")
     checkpoint = declared("tg_checkpoint.h", "TG_API")
-    assert len(kernel) >= 18 and len(engine) >= 23 and len(checkpoint) == 3
-    for name in kernel + engine + checkpoint:
+    events = declared("tg_events.h", "TG_API")
+    assert len(kernel) >= 23 and len(engine) >= 23 and len(checkpoint) == 3 and len(events) == 7
+    for name in kernel + engine + checkpoint + events:
         assert hasattr(lib, name), name
+    assert set(events) == set(bridge.EVENTS_ABI)
     assert set(kernel) == set(bridge.KERNEL_ABI)
     assert set(engine) == set(bridge.ENGINE_ABI)
     assert set(checkpoint) == set(bridge.CHECKPOINT_ABI)

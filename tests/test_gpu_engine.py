@@ -238,6 +238,52 @@ def test_host_program_trains_and_resumes(orc, tmp_path):
     assert a["step"] == b["step"] == 12
 
 
+def test_host_program_logs_a_run(orc, tmp_path):
+    """--log-to: TensorBoard events whose framing and payloads parse (the parser of tests/test_events.py) and a
+    report.json with the loss averaged over the last 1 % of the steps (loss_summary.cpp:5-29), for the
+    reference's own width-16 network (--width16 1, through tg_create) with four batches in flight."""
+    import json
+    import struct
+    import subprocess
+    from test_events import fields, one, records
+    from turbogpt_amd import build as native
+    data = tmp_path / "bytes.bin"
+    data.write_bytes(orc.fill_zipf_bytes(1 << 16, 9).tobytes())
+    run_dir = tmp_path / "runs" / "w16"
+    steps, batch, context = 300, 64, 8
+    done = subprocess.run([str(native.HOST_PROGRAM), "--data", str(data), "--width16", "1", "--depth", "4", "--context",
+                           str(context), "--batch", str(batch), "--chunk", "50", "--tokens", str(steps * batch * context),
+                           "--inflight", "4", "--log-to", str(run_dir), "--save", str(tmp_path / "w16.pt")],
+                          capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stderr
+    lines = [json.loads(line) for line in done.stdout.splitlines()]
+    assert [r["step"] for r in lines[:-1]] == [50, 100, 150, 200, 250, 300]
+    assert lines[-2]["loss"] < lines[0]["loss"] - 0.3  # it learns the Zipf byte frequencies
+    report = json.loads((run_dir / "report.json").read_text())
+    assert report["architecture"] == "swiglu48-rmsnorm-rope" and report["optimizer"] == "muon"
+    assert report["parameters"] == 21648 and report["steps"] == steps and report["tokens"] == steps * batch * context
+    assert report["final_loss_batches"] == 3 and len(report["position_bpb"]) == context  # last ceil(300 / 100) steps
+    assert report["final_bpb"] == pytest.approx(report["final_loss"] / np.log(2), rel=1e-6)
+    assert abs(report["final_loss"] * context - sum(report["position_bpb"]) * np.log(2) * 1.0) < 50  # finite numbers
+    assert report["max_staleness"] == 3 and 2.9 < report["mean_staleness"] <= 3.0
+    (event_file,) = list(run_dir.glob("events.out.tfevents.*"))
+    payloads = records(event_file)
+    scalars = {}
+    for payload in payloads[1:]:
+        event = fields(payload)
+        value = fields(one(fields(one(event, 5)), 1))
+        tensor = fields(one(value, 8))
+        if one(tensor, 1) == 1:
+            scalars.setdefault(one(value, 1).decode(), []).append((one(event, 2), struct.unpack("<f", one(tensor, 5))[0]))
+    assert [step for step, _ in scalars["loss"]] == [n * batch * context for n in (50, 100, 150, 200, 250, 300)]
+    assert scalars["loss"][-1][1] == pytest.approx(lines[-2]["loss"], abs=1e-5)
+    assert scalars["bits-per-byte"][-1][1] == pytest.approx(scalars["last_loss"][-1][1] / np.log(2), rel=1e-6)
+    assert scalars["model_bytes"] == [(0, 21648 * 4.0)] and scalars["lr"][-1][1] < scalars["lr"][1][1]
+    from turbogpt_amd.bridge import read_checkpoint
+    saved = read_checkpoint(tmp_path / "w16.pt")
+    assert saved["step"] == steps and saved["weights"].size == 21648 and saved["final_loss_batches"] == 3
+
+
 def test_engine_error_paths(orc):
     cfg = ModelConfig(d_model=128, depth=1, context=128, batch=1)
     with Native(cfg) as engine:

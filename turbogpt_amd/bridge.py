@@ -127,6 +127,16 @@ CHECKPOINT_ABI = {
     "tg_checkpoint_inspect": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
     "tg_checkpoint_read": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
 }
+# every symbol include/tg_events.h declares
+EVENTS_ABI = {
+    "tg_events_open": (vp, [C.c_char_p, C.c_char_p]),
+    "tg_events_path": (C.c_char_p, [vp]),
+    "tg_events_scalar": (i32, [vp, C.c_char_p, C.c_double, i64]),
+    "tg_events_text": (i32, [vp, C.c_char_p, C.c_char_p, i64]),
+    "tg_events_flush": (i32, [vp]),
+    "tg_events_close": (i32, [vp]),
+    "tg_crc32c": (C.c_uint32, [vp, sz]),
+}
 CLASSES = ("gemm_fwd", "gemm_dgrad", "gemm_wgrad", "attn_fwd", "attn_bwd", "layernorm_fwd", "layernorm_bwd",
            "head", "other", "optimizer")
 
@@ -144,7 +154,7 @@ def library():
             raise RuntimeError(f"{path} is missing: build it with `python -m turbogpt_amd.build` "
                                "(there is no CPU or PyTorch fallback)")
         lib = C.CDLL(str(path))
-        for name, (restype, argtypes) in {**KERNEL_ABI, **ENGINE_ABI, **CHECKPOINT_ABI}.items():
+        for name, (restype, argtypes) in {**KERNEL_ABI, **ENGINE_ABI, **CHECKPOINT_ABI, **EVENTS_ABI}.items():
             fn = getattr(lib, name)  # AttributeError if the symbol is not exported
             fn.restype, fn.argtypes = restype, argtypes
         _LIB = lib

@@ -331,14 +331,23 @@ std::string record_name(const std::string &prefix, int storage) {
     return prefix + "/data/" + std::to_string(storage);
 }
 
+// Elements of weights / momentum / variance.  Width 16 with 4 heads and a 48-wide MLP is the reference's own
+// network, whose flat layout is model.h:12-37 (no positions, no biases); every other shape is the wide
+// model of include/tg_model.h.
+int64_t expected_parameters(const TgModelConfig &m) {
+    if (m.d_model == 16 && m.heads == 4 && m.vocab == 256 && m.ffn == 48)
+        return 2 * 256 * 16 + 16 + int64_t(m.base.depth) * (2 * 16 + 4 * 48 * 16 + 16 * 16);
+    return tg_parameter_layout(&m).count;
+}
+
 void check_for_writing(const TgCheckpoint &c) {
     const TgModelConfig &m = c.model;
     if (m.base.depth < 1 || m.base.context < 1 || m.d_model < 1 || m.heads < 1 || m.vocab < 1 || m.ffn < 1)
         fail("model fields must be positive");
-    TgParameterLayout layout = tg_parameter_layout(&m);
-    if (m.base.depth > TG_MAX_DEPTH || layout.count != c.parameter_count)
+    const int64_t expected = m.base.depth > TG_MAX_DEPTH ? -1 : expected_parameters(m);
+    if (expected != c.parameter_count)
         fail("parameter_count " + std::to_string(c.parameter_count) + " does not match the model (" +
-             std::to_string(layout.count) + ")");
+             std::to_string(expected) + ")");
     if (!c.weights || !c.momentum || !c.variance)
         fail("weights, momentum and variance are required");
     if (c.final_loss_positions != 0 && c.final_loss_positions != m.base.context)
@@ -418,7 +427,7 @@ std::string read_header(const ZipReader &zip, TgCheckpoint &c) {
     std::memset(&c.model, 0, sizeof c.model);
     c.model.base.depth = int(s.depth), c.model.base.context = int(s.context);
     c.model.d_model = int(s.d_model), c.model.heads = int(s.heads), c.model.vocab = int(s.vocab), c.model.ffn = int(s.ffn);
-    c.parameter_count = tg_parameter_layout(&c.model).count;
+    c.parameter_count = expected_parameters(c.model);
     if (zip.find(record_name(prefix, S_WEIGHTS)).size != uint64_t(c.parameter_count) * 4 ||
         zip.find(record_name(prefix, S_MOMENTUM)).size != uint64_t(c.parameter_count) * 4 ||
         zip.find(record_name(prefix, S_VARIANCE)).size != uint64_t(c.parameter_count) * 4)
