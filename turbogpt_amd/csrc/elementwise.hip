@@ -481,13 +481,18 @@ __global__ __launch_bounds__(256) void sample_batch_kernel(const uint8_t *__rest
 __global__ __launch_bounds__(256) void position_means_kernel(const float *__restrict__ token_loss,
                                                              int batch, int context,
                                                              float *__restrict__ out) {
-    const int p = blockIdx.x * 256 + threadIdx.x;
+    // one wave per position: a lane sums every 64th sequence, then the lanes are folded in a fixed tree
+    const int p = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (p >= context)
         return;
     double sum = 0;
-    for (int b = 0; b < batch; ++b)
+    for (int b = lane; b < batch; b += 64)
         sum += token_loss[size_t(b) * context + p];
-    out[p] = float(sum / batch);
+#pragma unroll
+    for (int k = 32; k; k >>= 1)
+        sum += __shfl_xor(sum, k, 64);
+    if (lane == 0)
+        out[p] = float(sum / batch);
 }
 
 // ---- batched bf16 transposes ------------------------------------------------------------------
@@ -759,7 +764,7 @@ extern "C" int tgk_position_means(hipStream_t stream, const float *token_loss, i
                                   float *out) {
     return guarded([&] {
         require(token_loss && out && batch > 0 && context > 0, "position_means: missing operand");
-        hipLaunchKernelGGL(position_means_kernel, dim3((context + 255) / 256), dim3(256), 0, stream, token_loss,
+        hipLaunchKernelGGL(position_means_kernel, dim3((context + 3) / 4), dim3(256), 0, stream, token_loss,
                            batch, context, out);
         check_hip(hipGetLastError(), "position_means launch: ");
     });

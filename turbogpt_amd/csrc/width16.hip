@@ -585,30 +585,52 @@ struct Jobs {
     Job job[MAX_JOBS];
     int count;
 };
-// partial[chunk][offset + o*in + i] = sum over the chunk's tokens, in token order
+// partial[chunk][offset + o*in + i] = sum over the chunk's tokens, in token order.  A thread owns output row o
+// and a 16-wide slab of inputs: per token it reads one dy value and one 32-byte row piece that every thread of
+// the same slab shares, and keeps 16 sums in registers.  (The widest jobs, head and embedding, are 256 x 16.)
 __global__ __launch_bounds__(256) void w16_weight_gradient_kernel(Jobs jobs, int tokens, int parameters, float *partials) {
     const Job &job = jobs.job[blockIdx.y];
     const int first = blockIdx.x * CHUNK, last = min(first + CHUNK, tokens);
-    float *out = partials + size_t(blockIdx.x) * parameters + job.offset;
-    for (int e = threadIdx.x; e < job.out * job.in; e += 256) {
-        const int o = e / job.in, i = e - o * job.in;
-        float acc = 0.f;
-        if (job.kind == JOB_OUTER) {
-            const bf16_t *dy = static_cast<const bf16_t *>(job.dy);
-            for (int t = first; t < last; ++t)
-                acc = fmaf(bf16_to_float(dy[size_t(t) * job.ld_dy + o]), bf16_to_float(job.x[size_t(t) * job.ld_x + i]), acc);
-        } else if (job.kind == JOB_COLUMN_SUM) {
-            const float *gz = static_cast<const float *>(job.dy);
-            for (int t = first; t < last; ++t)
-                acc += gz[size_t(t) * W + i];
-        } else {
-            const uint8_t *ids = static_cast<const uint8_t *>(job.dy);
-            for (int t = first; t < last; ++t)
-                if (ids[t] == o)
-                    acc += bf16_to_float(job.x[size_t(t) * W + i]);
+    const int slabs = job.in >> 4, o = threadIdx.x / slabs, slab = threadIdx.x - o * slabs;
+    if (o >= job.out)
+        return;
+    float acc[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k)
+        acc[k] = 0.f;
+    if (job.kind == JOB_OUTER) {
+        const bf16_t *dy = static_cast<const bf16_t *>(job.dy) + o;
+        const bf16_t *x = job.x + slab * 16;
+        for (int t = first; t < last; ++t) {
+            const float d = bf16_to_float(dy[size_t(t) * job.ld_dy]);
+            float v[16];
+            load_row16(x + size_t(t) * job.ld_x, v);
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                acc[k] = fmaf(d, v[k], acc[k]);
         }
-        out[e] = acc;
+    } else if (job.kind == JOB_COLUMN_SUM) {
+        const float *gz = static_cast<const float *>(job.dy);
+        for (int t = first; t < last; ++t)
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                acc[k] += gz[size_t(t) * W + k];
+    } else {
+        const uint8_t *ids = static_cast<const uint8_t *>(job.dy);
+        for (int t = first; t < last; ++t) {
+            if (ids[t] != o)
+                continue;
+            float v[16];
+            load_row16(job.x + size_t(t) * W, v);
+#pragma unroll
+            for (int k = 0; k < 16; ++k)
+                acc[k] += v[k];
+        }
     }
+    float *out = partials + size_t(blockIdx.x) * parameters + job.offset + o * job.in + slab * 16;
+#pragma unroll
+    for (int k = 0; k < 16; k += 4)
+        *reinterpret_cast<f32x4 *>(out + k) = f32x4{acc[k], acc[k + 1], acc[k + 2], acc[k + 3]};
 }
 __global__ __launch_bounds__(256) void w16_fold_kernel(const float *__restrict__ partials, int chunks, int parameters,
                                                        float *gradient) {
