@@ -39,8 +39,9 @@ TGK_API int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint16_t
                  uint16_t *gelu_out, int ldg);
 
 /* The same forward projection with the weight given transposed, Wt[K][N] (leading dimension ldwt):
- * the copy engine then moves whole rows of Wt instead of 64-byte pieces of W, which is markedly
- * faster on the wide projections.  Same epilogues and shape rules as tgk_gemm_fwd. */
+ * whole rows of Wt are copied instead of 64-byte pieces of W, which is faster where tgk_gemm_fwd cannot
+ * use its 64-k stages (K not a multiple of 64, or N not a multiple of 192).  Same epilogues and shape
+ * rules as tgk_gemm_fwd. */
 TGK_API int tgk_gemm_fwd_t(hipStream_t stream, int M, int N, int K, const uint16_t *X, int ldx,
                            const uint16_t *Wt, int ldwt, uint16_t *Y, int ldy, const uint16_t *residual,
                            int ldr, uint16_t *gelu_out, int ldg);
@@ -54,6 +55,14 @@ TGK_API int tgk_gemm_fwd_t(hipStream_t stream, int M, int N, int K, const uint16
 TGK_API int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uint16_t *dY, int lddy,
                    const uint16_t *W, int ldw, uint16_t *dX, int lddx, const uint16_t *gelu_pre,
                    int ldu);
+
+/* The same input gradient with the weight given transposed, Wt[K][N] (leading dimension ldwt): both
+ * operands are then contiguous along the reduced dimension and the product runs on the forward
+ * kernel (64-k stages when N is a multiple of 64 and K of 192).  Same epilogue and shape rules as
+ * tgk_gemm_dgrad. */
+TGK_API int tgk_gemm_dgrad_t(hipStream_t stream, int M, int N, int K, const uint16_t *dY, int lddy,
+                             const uint16_t *Wt, int ldwt, uint16_t *dX, int lddx,
+                             const uint16_t *gelu_pre, int ldu);
 
 /* Weight gradient, replaces weight_gradient (cuda/ops.cuh:83-109) and, through its fixed-order
  * split-K reduction, reduce_gradients (cuda/trainer.cuh:9-47).

@@ -20,6 +20,7 @@ KERNEL_ABI = {
     "tgk_gemm_fwd_t": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
     "tgk_transpose_batch": (i32, [vp, vp, vp, vp, i32, i32]),
     "tgk_gemm_dgrad": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
+    "tgk_gemm_dgrad_t": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
     "tgk_gemm_wgrad": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, i32, vp, sz]),
     "tgk_gemm_wgrad_workspace": (sz, [i32, i32, i32]),
     "tgk_attn_fwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, f32]),

@@ -197,7 +197,8 @@ struct Engine {
             (void)hipStreamDestroy(stream);
     }
 
-    // forward projections read the transposed weights: call after every change of a version's hi half
+    // input gradients and the head's forward projection read the transposed weights: call after every change of a
+    // version's hi half
     void refresh_transposed(const Version &v) {
         if (width16)
             return;
@@ -230,14 +231,14 @@ struct Engine {
             LayerBuffers &b = layers[l];
             OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, x[l], w(p.ln1_g), wl(p.ln1_g), w(p.ln1_b), wl(p.ln1_b), b.n1,
                                  config.ln_eps));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, 3 * d, d, b.n1, d, wt(p.qkv), 3 * d, b.qkv, 3 * d, nullptr, 0, nullptr, 0));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, 3 * d, d, b.n1, d, w(p.qkv), d, b.qkv, 3 * d, nullptr, 0, nullptr, 0));
             OP(TG_CLASS_ATTN_FWD, tgk_attn_fwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
                             3 * d, b.o, d, b.lse, scale));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, d, d, b.o, d, wt(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, d, b.o, d, w(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
             OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, b.mid, w(p.ln2_g), wl(p.ln2_g), w(p.ln2_b), wl(p.ln2_b), b.n2,
                                  config.ln_eps));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, F, d, b.n2, d, wt(p.mlp_up), F, b.u, F, nullptr, 0, b.a, F));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd_t(stream, M, d, F, b.a, F, wt(p.mlp_down), d, x[l + 1], d, b.mid, d, nullptr, 0));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, F, d, b.n2, d, w(p.mlp_up), d, b.u, F, nullptr, 0, b.a, F));
+            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, F, b.a, F, w(p.mlp_down), F, x[l + 1], d, b.mid, d, nullptr, 0));
         }
         OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, x[c.depth], w(layout.lnf_g), wl(layout.lnf_g), w(layout.lnf_b),
                              wl(layout.lnf_b), nf, config.ln_eps));
@@ -260,6 +261,7 @@ struct Engine {
         }
         const auto w = [&](int64_t offset) { return v.hi + offset; };
         const auto wl = [&](int64_t offset) { return v.lo + offset; };
+        const auto wt = [&](int64_t offset) { return v.t + offset; };
         std::vector<bf16_t *> &x = s.x;
         std::vector<LayerBuffers> &layers = s.layers;
         bf16_t *nf = s.nf, *logits = s.logits, *dh = s.dh, *t1 = s.t1, *du = s.du, *dqkv = s.dqkv;
@@ -267,26 +269,26 @@ struct Engine {
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
         float *g = gradient;
         OP(TG_CLASS_HEAD, tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
-        OP(TG_CLASS_HEAD, tgk_gemm_dgrad(stream, M, V, d, logits, V, w(layout.head), d, t1, d, nullptr, 0));
+        OP(TG_CLASS_HEAD, tgk_gemm_dgrad_t(stream, M, V, d, logits, V, wt(layout.head), V, t1, d, nullptr, 0));
         OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, x[c.depth], t1, w(layout.lnf_g), wl(layout.lnf_g), dh,
                              g + layout.lnf_g, g + layout.lnf_b, config.ln_eps, 0, 0, workspace, workspace_bytes));
         for (int l = c.depth - 1; l >= 0; --l) {
             const TgLayerParameters &p = layout.layers[l];
             LayerBuffers &b = layers[l];
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, F, dh, d, b.a, F, g + p.mlp_down, F, 0, workspace, workspace_bytes));
-            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, d, F, dh, d, w(p.mlp_down), F, du, F, b.u, F));
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, F, d, du, F, b.n2, d, g + p.mlp_up, d, 0, workspace, workspace_bytes));
-            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, F, d, du, F, w(p.mlp_up), d, t1, d, nullptr, 0));
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, du, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
             OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, b.mid, t1, w(p.ln2_g), wl(p.ln2_g), dh, g + p.ln2_g, g + p.ln2_b,
                                  config.ln_eps, 1, 0, workspace, workspace_bytes));
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, d, dh, d, b.o, d, g + p.attn_out, d, 0, workspace, workspace_bytes));
-            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, d, d, dh, d, w(p.attn_out), d, t1, d, nullptr, 0));
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, d, dh, d, wt(p.attn_out), d, t1, d, nullptr, 0));
             OP(TG_CLASS_ATTN_BWD, tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
                             3 * d, b.o, d, b.lse, t1, d, dqkv, dqkv + d, dqkv + 2 * d, 3 * d, scale, workspace,
                             workspace_bytes));
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, 3 * d, d, dqkv, 3 * d, b.n1, d, g + p.qkv, d, 0, workspace,
                               workspace_bytes));
-            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad(stream, M, 3 * d, d, dqkv, 3 * d, w(p.qkv), d, t1, d, nullptr, 0));
+            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, 3 * d, d, dqkv, 3 * d, wt(p.qkv), 3 * d, t1, d, nullptr, 0));
             OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, x[l], t1, w(p.ln1_g), wl(p.ln1_g), dh, g + p.ln1_g, g + p.ln1_b,
                                  config.ln_eps, 1, 0, workspace, workspace_bytes));
         }

@@ -89,6 +89,63 @@ struct EpilogueF32 {
     }
 };
 
+// bf16 outputs: each 32x32 accumulator tile is rounded and transposed through a wave-private LDS buffer
+// (32 rows of 64 bytes, 16-byte chunk c of row r at c ^ ((r >> 2) & 3)), so that a lane finishes 8
+// consecutive n of rows get_row and get_row + 16.  LDS operations of one wave execute in order, so no
+// barrier is needed around the buffer.
+template <int FM, int FN, class Epilogue, class Aux>
+TG_DEVICE void staged_store_bf16(const f32x16 (&acc)[FM][FN], const Aux &aux, unsigned char *mine,
+                                 const Epilogue &epilogue, int m_base, int n_base, int lane) {
+    const int get_row = lane >> 2, get_chunk = lane & 3;
+    const int row = lane & 31;
+    unsigned char *put = mine + row * 64 + (lane >> 5) * 8;
+    const int put_swizzle = (row >> 2) & 3;
+    // rows r and r + 16 share a swizzle term, so the second half is 1 KiB further on
+    const unsigned char *get = mine + get_row * 64 + ((get_chunk ^ ((get_row >> 2) & 3)) << 4);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int m = m_base + i * 32 + get_row, n = n_base + j * 32 + get_chunk * 8;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                u32x2 packed;
+                packed.x = pack_bf16(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
+                packed.y = pack_bf16(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+                *reinterpret_cast<u32x2 *>(put + ((q ^ put_swizzle) << 4)) = packed;
+            }
+            epilogue.finish(m, n, *reinterpret_cast<const u32x4 *>(get), aux[i][j][0]);
+            epilogue.finish(m + 16, n, *reinterpret_cast<const u32x4 *>(get + 1024), aux[i][j][1]);
+        }
+}
+
+// fp32 outputs: the same through a buffer of 32 rows of 128 bytes (16-byte chunk c of row r at c ^ ((r >> 1) & 7));
+// a lane finishes 4 consecutive n, 8 lanes cover a 128-byte row piece.
+template <int FM, int FN, class Epilogue>
+TG_DEVICE void staged_store_f32(const f32x16 (&acc)[FM][FN], unsigned char *mine, const Epilogue &epilogue,
+                                int m_base, int n_base, int lane, int split) {
+    const int row = lane & 31;
+    unsigned char *put = mine + row * 128;
+    const int put_swizzle = (row >> 1) & 7, g = lane >> 5;
+    const int first_row = lane >> 3, chunk = lane & 7;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const f32x4 v = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+                *reinterpret_cast<f32x4 *>(put + (((2 * q + g) ^ put_swizzle) << 4)) = v;
+            }
+#pragma unroll
+            for (int part = 0; part < 4; ++part) {
+                const int r = first_row + part * 8;
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(mine + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4));
+                epilogue.finish(m_base + i * 32 + r, n_base + j * 32 + chunk * 4, v, split);
+            }
+        }
+}
+
 constexpr int BK = 32;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -334,54 +391,223 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
             c_slot = next_slot;
         }
         if constexpr (Epilogue::BF16) {
-            // wave-private buffer: 32 rows of 64 bytes, 16-byte chunk c of row r at c ^ ((r >> 2) & 3).
-            // LDS operations of one wave execute in order, so no barrier is needed around it.
-            unsigned char *mine = smem + S * STAGE + wave * 2048;
-            const int row = lane & 31;
-            unsigned char *put = mine + row * 64 + (lane >> 5) * 8;
-            const int put_swizzle = (row >> 2) & 3;
-            // rows r and r + 16 share a swizzle term, so the second half is 1 KiB further on
-            const unsigned char *get = mine + get_row * 64 + ((get_chunk ^ ((get_row >> 2) & 3)) << 4);
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    const int m = m0 + wm + i * 32 + get_row, n = n0 + wn + j * 32 + get_chunk * 8;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        u32x2 packed;
-                        packed.x = pack_bf16(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1]);
-                        packed.y = pack_bf16(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
-                        *reinterpret_cast<u32x2 *>(put + ((q ^ put_swizzle) << 4)) = packed;
-                    }
-                    epilogue.finish(m, n, *reinterpret_cast<const u32x4 *>(get), aux[i][j][0]);
-                    epilogue.finish(m + 16, n, *reinterpret_cast<const u32x4 *>(get + 1024), aux[i][j][1]);
-                }
+            staged_store_bf16<FM, FN>(acc, aux, smem + S * STAGE + wave * 2048, epilogue, m0 + wm, n0 + wn, lane);
         } else {
-            // wave-private buffer: 32 rows of 128 bytes, 16-byte chunk c of row r at c ^ ((r >> 1) & 7)
-            unsigned char *mine = smem + S * STAGE + wave * 4096;
-            const int row = lane & 31;
-            unsigned char *put = mine + row * 128;
-            const int put_swizzle = (row >> 1) & 7, g = lane >> 5;
-            const int first_row = lane >> 3, chunk = lane & 7;
+            staged_store_f32<FM, FN>(acc, smem + S * STAGE + wave * 4096, epilogue, m0 + wm, n0 + wn, lane, split);
+        }
+    }
+    wait_vmcnt<0>();
+}
+
+// ---- 64 k per stage, two stages --------------------------------------------------------------------
+// k-contiguous tile of ROWS rows x 64 k: 128-byte rows (every copy request is a whole cache line), 16-byte
+// chunk c of row r stored at chunk c ^ ((r >> 1) & 7): conflict-free for ds_read_b128 with 64 banks.
+template <int ROWS> struct TileKC64 {
+    static constexpr int LOADS = ROWS * 128 / 4096; // wave-wide copies per thread per stage
+    static constexpr int BYTES = ROWS * 128;
+    TG_DEVICE static int64_t step(int) { return 64; } // elements from one stage to the next
+    TG_DEVICE static int64_t origin(int row0, int k0, int ld) { return int64_t(row0) * ld + k0; }
+    TG_DEVICE static int64_t source_offset(int j, int tid, int ld) {
+        const int wave = tid >> 6, lane = tid & 63;
+        const int row = (j * 4 + wave) * 8 + (lane >> 3), phys = lane & 7;
+        const int chunk = phys ^ ((row >> 1) & 7);
+        return int64_t(row) * ld + chunk * 8;
+    }
+    TG_DEVICE static uint32_t lds_offset(int j, int tid) { return uint32_t((j * 4 + (tid >> 6)) * 1024); }
+    // fragment for rows row0 + lane%32, 16-k step ks of the stage (0..3): k = ks*16 + 8*(lane/32) .. +7
+    TG_DEVICE static bf16x8 frag(const unsigned char *tile, int row0, int ks, int lane) {
+        const int row = row0 + (lane & 31), chunk = (ks * 2 + (lane >> 5)) ^ ((row >> 1) & 7);
+        return *reinterpret_cast<const bf16x8 *>(tile + row * 128 + chunk * 16);
+    }
+};
+// k-strided tile: 64 k-rows x ROWS columns in the natural [k][row] image, swizzled and read like TileKS
+template <int ROWS> struct TileKS64 {
+    static constexpr int LOADS = ROWS * 128 / 4096;
+    static constexpr int BYTES = ROWS * 128;
+    static constexpr int CHUNKS_PER_ROW = ROWS / 8;
+    TG_DEVICE static int64_t step(int ld) { return int64_t(64) * ld; }
+    TG_DEVICE static int64_t origin(int row0, int k0, int ld) { return int64_t(k0) * ld + row0; }
+    TG_DEVICE static int64_t source_offset(int j, int tid, int ld) {
+        const int wave = tid >> 6, lane = tid & 63;
+        const int q = (j * 4 + wave) * 64 + lane, r = q / CHUNKS_PER_ROW, p = q - r * CHUNKS_PER_ROW;
+        const int chunk = p ^ TileKS<ROWS>::swizzle(r);
+        return int64_t(r) * ld + chunk * 8;
+    }
+    TG_DEVICE static uint32_t lds_offset(int j, int tid) { return uint32_t((j * 4 + (tid >> 6)) * 1024); }
+    TG_DEVICE static bf16x8 frag(const unsigned char *tile, int row0, int ks, int lane) {
+        return TileKS<ROWS>::frag(tile, row0, ks, lane); // k-rows ks*16 .. of the 64
+    }
+};
+template <int ROWS, bool KC> struct Tile64Of;
+template <int ROWS> struct Tile64Of<ROWS, true> { using type = TileKC64<ROWS>; };
+template <int ROWS> struct Tile64Of<ROWS, false> { using type = TileKS64<ROWS>; };
+
+// The same product as gemm_kernel with two 64-k stages of (BM + BN) * 128 bytes: per stage one wait, one barrier,
+// and the copies of the next stage issued one behind every second MFMA.  A copy instruction that finds the
+// vector-memory queue full stalls its wave, and with it the wave's MFMAs; kept apart, the copies overlap them
+// (measured: 6-8 % over issuing the ten copies in a burst, on every training shape).  k-contiguous operands are
+// copied in whole 128-byte lines and read with ds_read_b128.  The epilogue's transposition buffers lie in the
+// stage consumed last; the stage being filled is the other one.  The reduced dimension is a multiple of 64.
+template <int BM, int BN, bool AKC, bool BKC, class Epilogue>
+__global__ __launch_bounds__(256, 2) void gemm64_kernel(const bf16_t *__restrict__ A, int lda,
+                                                      const bf16_t *__restrict__ B, int ldb, int k_chunks,
+                                                      int splits, int tiles_n, int tiles_total, int xcd_cols,
+                                                      Epilogue epilogue) {
+    using TA = typename Tile64Of<BM, AKC>::type;
+    using TB = typename Tile64Of<BN, BKC>::type;
+    constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+    constexpr int LA = TA::LOADS, LB = TB::LOADS, LOADS = LA + LB;
+    constexpr int SLOT = TA::BYTES + TB::BYTES;
+    static_assert(LOADS * 2 <= FM * FN * 4, "copies are paired with the MFMAs of one stage");
+    static_assert(4 * (Epilogue::BF16 ? 2048 : 4096) <= SLOT, "the epilogue buffers fit one stage");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t smem_base = lds_address(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    const int items = tiles_total * splits, stride = gridDim.x;
+
+    // Same placement as gemm_kernel: item i belongs to XCD i % 8 and is that XCD's (i / 8)-th item; without
+    // split-K the tile grid is cut into (8 / xcd_cols) x xcd_cols rectangles, one per XCD.
+    auto locate = [&](int item, int &m0, int &n0, int &c0, int &nc) {
+        int split = 0, tile_m, tile_n;
+        if ((items & 7) == 0 && xcd_cols > 1) {
+            const int xcd = item & 7, index = item >> 3;
+            const int cols = tiles_n / xcd_cols, rows = (tiles_total / tiles_n) / (8 / xcd_cols);
+            tile_m = (xcd / xcd_cols) * rows + index / cols;
+            tile_n = (xcd % xcd_cols) * cols + index % cols;
+        } else {
+            int logical = item;
+            if ((items & 7) == 0)
+                logical = (item & 7) * (items >> 3) + (item >> 3);
+            split = logical / tiles_total;
+            const int tile = logical - split * tiles_total;
+            tile_m = tile / tiles_n;
+            tile_n = tile % tiles_n;
+        }
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
+        c0 = split * k_chunks / splits;
+        nc = (split + 1) * k_chunks / splits - c0;
+        return split;
+    };
+
+    // ---- producer: the stage after the one being consumed ------------------------------------------
+    int p_item = blockIdx.x, p_left = 0, p_slot = 0;
+    const bf16_t *pa[LA], *pb[LB];
+    const int64_t a_step = TA::step(lda), b_step = TB::step(ldb);
+    auto producer_open = [&]() {
+        int m0, n0, c0, nc;
+        locate(p_item, m0, n0, c0, nc);
+        p_left = nc;
+        const bf16_t *a0 = A + TA::origin(m0, c0 * 64, lda), *b0 = B + TB::origin(n0, c0 * 64, ldb);
+#pragma unroll
+        for (int j = 0; j < LA; ++j)
+            pa[j] = a0 + TA::source_offset(j, tid, lda);
+#pragma unroll
+        for (int j = 0; j < LB; ++j)
+            pb[j] = b0 + TB::source_offset(j, tid, ldb);
+    };
+    auto copy_one = [&](int n) { // n-th of the LOADS copies of a stage, into slot p_slot
+        const uint32_t to = smem_base + uint32_t(p_slot) * SLOT;
+        if (n < LA) {
+            async_copy16(__builtin_amdgcn_readfirstlane(to + TA::lds_offset(n, tid)), pa[n]);
+            pa[n] += a_step;
+        } else {
+            async_copy16(__builtin_amdgcn_readfirstlane(to + TA::BYTES + TB::lds_offset(n - LA, tid)), pb[n - LA]);
+            pb[n - LA] += b_step;
+        }
+    };
+    if (p_item >= items)
+        return;
+    producer_open();
+#pragma unroll
+    for (int n = 0; n < LOADS; ++n)
+        copy_one(n);
+    --p_left;
+    p_slot = 1;
+
+    int c_slot = 0;
+    for (int item = blockIdx.x; item < items; item += stride) {
+        int m0, n0, c0, nc;
+        const int split = locate(item, m0, n0, c0, nc);
+        f32x16 acc[FM][FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[i][j][r] = 0.f;
+        const int get_row = lane >> 2, get_chunk = lane & 3;
+        u32x4 aux[Epilogue::BF16 ? FM : 1][Epilogue::BF16 ? FN : 1][2];
+        for (int c = 0; c < nc; ++c) {
+            wait_vmcnt<0>(); // this wave's copies of stage c (and the previous tile's stores) are done
+            __syncthreads(); // everyone's are, and everyone is done reading the other slot
+            if (Epilogue::BF16 && c == nc - 1 && epilogue.wants_aux()) {
+                // the epilogue's second input, in its row layout, lands while the last stage is multiplied
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+#pragma unroll
+                        for (int half = 0; half < 2; ++half)
+                            aux[Epilogue::BF16 ? i : 0][Epilogue::BF16 ? j : 0][half] = epilogue.load_aux(
+                                m0 + wm + i * 32 + get_row + half * 16, n0 + wn + j * 32 + get_chunk * 8);
+            }
+            bool copy = true;
+            if (p_left == 0) {
+                p_item += stride;
+                copy = p_item < items;
+                if (copy)
+                    producer_open();
+            }
+            const unsigned char *sa = smem + c_slot * SLOT, *sb = sa + TA::BYTES;
+            bf16x8 af[2][FM], bfr[2][FN];
 #pragma unroll
             for (int i = 0; i < FM; ++i)
+                af[0][i] = TA::frag(sa, wm + i * 32, 0, lane);
 #pragma unroll
-                for (int j = 0; j < FN; ++j) {
+            for (int j = 0; j < FN; ++j)
+                bfr[0][j] = TB::frag(sb, wn + j * 32, 0, lane);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const f32x4 v = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
-                                         acc[i][j][q * 4 + 3]};
-                        *reinterpret_cast<f32x4 *>(put + (((2 * q + g) ^ put_swizzle) << 4)) = v;
-                    }
+            for (int ks = 0; ks < 4; ++ks) {
+                if (ks < 3) {
 #pragma unroll
-                    for (int part = 0; part < 4; ++part) {
-                        const int r = first_row + part * 8;
-                        const f32x4 v = *reinterpret_cast<const f32x4 *>(mine + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4));
-                        epilogue.finish(m0 + wm + i * 32 + r, n0 + wn + j * 32 + chunk * 4, v, split);
-                    }
+                    for (int i = 0; i < FM; ++i)
+                        af[(ks + 1) & 1][i] = TA::frag(sa, wm + i * 32, ks + 1, lane);
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+                        bfr[(ks + 1) & 1][j] = TB::frag(sb, wn + j * 32, ks + 1, lane);
                 }
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ks & 1][j], af[ks & 1][i], acc[i][j], 0, 0, 0);
+                        const int q = ks * FM * FN + i * FN + j; // MFMA number within the stage
+                        if ((q & 1) && (q >> 1) < LOADS) {
+                            __builtin_amdgcn_sched_barrier(0);
+                            if (copy)
+                                copy_one(q >> 1);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+            }
+            if (copy) {
+                --p_left;
+                p_slot ^= 1;
+            }
+            c_slot ^= 1;
         }
+        // The transposition buffers lie in the stage consumed last (c_slot ^ 1 now); other waves may still be
+        // reading fragments there.
+        __syncthreads();
+        unsigned char *slot = smem + (c_slot ^ 1) * SLOT;
+        if constexpr (Epilogue::BF16)
+            staged_store_bf16<FM, FN>(acc, aux, slot + wave * 2048, epilogue, m0 + wm, n0 + wn, lane);
+        else
+            staged_store_f32<FM, FN>(acc, slot + wave * 4096, epilogue, m0 + wm, n0 + wn, lane, split);
     }
     wait_vmcnt<0>();
 }
@@ -505,6 +731,31 @@ void dispatch_gemm(hipStream_t stream, Tile tile, const bf16_t *A, int lda, cons
         launch_gemm<128, 128, 4, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, blocks, epilogue);
 }
 
+// 128x192 tiles with the reduced dimension a multiple of 64 take the two-stage 64-k kernel.
+bool takes_64(Tile tile, int reduced) { return tile == TILE_128x192 && reduced % 64 == 0; }
+
+template <bool AKC, bool BKC, class Epilogue>
+void launch_gemm64(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
+                   int splits, const Epilogue &epilogue) {
+    constexpr int BM = 128, BN = 192;
+    auto kernel = gemm64_kernel<BM, BN, AKC, BKC, Epilogue>;
+    constexpr size_t lds = 2 * (BM + BN) * 128;
+    static std::atomic<bool> configured[MAX_DEVICES];
+    const int device = current_device();
+    if (!configured[device].load(std::memory_order_acquire)) {
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)),
+                  "gemm LDS size: ");
+        configured[device].store(true, std::memory_order_release);
+    }
+    const int tiles_m = M / BM, tiles_n = N / BN, tiles = tiles_m * tiles_n, items = tiles * splits;
+    const int max_blocks = resident_blocks(TILE_128x192);
+    const int blocks = items < max_blocks ? items : max_blocks;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, A, lda, B, ldb, K / 64, splits, tiles_n, tiles,
+                       splits == 1 ? xcd_columns(tiles_m, tiles_n, BM, BN, K, blocks) : 1, epilogue);
+    check_hip(hipGetLastError(), "gemm launch: ");
+}
+
 void check_operand(const void *p, int ld, const char *name) {
     if (!p || (reinterpret_cast<uintptr_t>(p) & 15) || ld % 8)
         throw std::invalid_argument(std::string("gemm operand ") + name +
@@ -542,7 +793,10 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
             check_operand(gelu_out, ldg, "gelu_out");
             e.out2 = gelu_out, e.ld_out2 = ldg, e.mode = EPI_GELU;
         }
-        dispatch_gemm<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, 1, e);
+        if (takes_64(tile, K))
+            launch_gemm64<true, true>(stream, X, ldx, W, ldw, M, N, K, 1, e);
+        else
+            dispatch_gemm<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, 1, e);
     });
 }
 
@@ -592,6 +846,30 @@ extern "C" int tgk_gemm_dgrad(hipStream_t stream, int M, int N, int K, const uin
     });
 }
 
+extern "C" int tgk_gemm_dgrad_t(hipStream_t stream, int M, int N, int K, const uint16_t *dY, int lddy,
+                                const uint16_t *Wt, int ldwt, uint16_t *dX, int lddx,
+                                const uint16_t *gelu_pre, int ldu) {
+    return guarded([&] {
+        require(M > 0 && N > 0 && K > 0, "gemm_dgrad_t: empty shape");
+        require(N % BK == 0, "gemm_dgrad_t: N (the reduced dimension) must be a multiple of 32");
+        const Tile tile = choose_tile(M, K);
+        require(tile != TILE_NONE, "gemm_dgrad_t: M must be a multiple of 128 and K of 128 or 192");
+        check_operand(dY, lddy, "dY");
+        check_operand(Wt, ldwt, "Wt");
+        check_operand(dX, lddx, "dX");
+        EpilogueBf16 e{dX, lddx, nullptr, 0, nullptr, 0, EPI_PLAIN};
+        if (gelu_pre) {
+            check_operand(gelu_pre, ldu, "gelu_pre");
+            e.aux = gelu_pre, e.ld_aux = ldu, e.mode = EPI_GELU_BWD;
+        }
+        // C[m][i] = sum_o dY[m][o] Wt[i][o]: the forward product with (rows, reduced) = (K, N)
+        if (takes_64(tile, N))
+            launch_gemm64<true, true>(stream, dY, lddy, Wt, ldwt, M, K, N, 1, e);
+        else
+            dispatch_gemm<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, 1, e);
+    });
+}
+
 extern "C" size_t tgk_gemm_wgrad_workspace(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0 || M % BK)
         return 0;
@@ -617,14 +895,20 @@ extern "C" int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uin
         const int splits = wgrad_splits(tile, (N / tile_rows(tile)) * (K / tile_cols(tile)), M / BK);
         if (splits == 1) {
             EpilogueF32 e{dW, lddw, 0, accumulate};
-            dispatch_gemm<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, 1, e);
+            if (takes_64(tile, M))
+                launch_gemm64<false, false>(stream, dY, lddy, X, ldx, N, K, M, 1, e);
+            else
+                dispatch_gemm<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, 1, e);
             return;
         }
         const size_t need = size_t(splits) * N * K * sizeof(float);
         require(workspace && workspace_bytes >= need && !(reinterpret_cast<uintptr_t>(workspace) & 15),
                 "gemm_wgrad: workspace too small (see tgk_gemm_wgrad_workspace)");
         EpilogueF32 e{static_cast<float *>(workspace), K, size_t(N) * K, 0};
-        dispatch_gemm<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, splits, e);
+        if (takes_64(tile, M))
+            launch_gemm64<false, false>(stream, dY, lddy, X, ldx, N, K, M, splits, e);
+        else
+            dispatch_gemm<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, splits, e);
         const size_t quads = size_t(N) * K / 4;
         const int blocks = int((quads + 255) / 256 < 4096 ? (quads + 255) / 256 : 4096);
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, stream,
