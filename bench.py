@@ -28,7 +28,7 @@ M = B * T
 ALGORITHMIC_BYTES_PER_LAUNCH = sum(2 * (M * k + n * k + M * n) for n, k in
                                    [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
 # HBM bytes per launch of that kernel, measured with rocprofv3 FETCH_SIZE / WRITE_SIZE runs of --traffic-probe
-HBM_TRAFFIC_PER_LAUNCH = 150.5e6
+HBM_TRAFFIC_PER_LAUNCH = 150.4e6
 
 
 def gemm_flops():
@@ -142,6 +142,8 @@ def kernel_sweeps(out):
                                                       y.data_ptr(), n, None, 0, None, 0)),
             "dgrad": lambda: check(lib.tgk_gemm_dgrad(stream, M, n, k, dy.data_ptr(), n, w.data_ptr(), k,
                                                       dx.data_ptr(), k, None, 0)),
+            "dgrad_t": lambda: check(lib.tgk_gemm_dgrad_t(stream, M, n, k, dy.data_ptr(), n, wt.data_ptr(), n,
+                                                          dx.data_ptr(), k, None, 0)),
             "wgrad": lambda: check(lib.tgk_gemm_wgrad(stream, M, n, k, dy.data_ptr(), n, x.data_ptr(), k,
                                                       dw.data_ptr(), k, 0, ws.data_ptr(), need)),
         }
@@ -176,8 +178,8 @@ def kernel_sweeps(out):
 def traffic_probe():
     """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: one plain copy of known size (256 MiB in,
     256 MiB out: the calibration dispatch) followed by one launch of each forward block projection
-    (on transposed weights, as the engine runs them) and of each dgrad - the eight uses per layer of
-    the kernel that `roofline` describes."""
+    and of each dgrad (on transposed weights), as the engine runs them - the eight uses per layer of the
+    kernel that `roofline` describes."""
     import torch
     from turbogpt_amd.bridge import check, library
     lib = library()
@@ -196,10 +198,9 @@ def traffic_probe():
         y = torch.empty(M, n, device="cuda", dtype=torch.bfloat16)
         dx = torch.empty(M, k, device="cuda", dtype=torch.bfloat16)
         torch.cuda.synchronize()
-        check(lib.tgk_gemm_fwd_t(stream, M, n, k, x.data_ptr(), k, wt.data_ptr(), n, y.data_ptr(), n, None, 0,
-                                 None, 0))
+        check(lib.tgk_gemm_fwd(stream, M, n, k, x.data_ptr(), k, w.data_ptr(), k, y.data_ptr(), n, None, 0, None, 0))
         torch.cuda.synchronize()
-        check(lib.tgk_gemm_dgrad(stream, M, n, k, dy.data_ptr(), n, w.data_ptr(), k, dx.data_ptr(), k, None, 0))
+        check(lib.tgk_gemm_dgrad_t(stream, M, n, k, dy.data_ptr(), n, wt.data_ptr(), n, dx.data_ptr(), k, None, 0))
         torch.cuda.synchronize()
     print(json.dumps({"probe": "traffic", "copy_bytes_each_way": 1 << 28,
                       "order": "per shape (K, N): forward, then dgrad", "shapes": shapes,
@@ -256,9 +257,9 @@ def main():
         rate = amount / (per_step_ms * 1e-3) / 1e12 if per_step_ms > 0 else 0.0
         classes[name] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // 3,
                          ("tflops" if kind == "flop" else "tb_per_s"): round(rate, 2)}
-    # dominant MFMA kernel: gemm_kernel<128,192,3,true,false,EpilogueBf16> - activations k-contiguous,
-    # weights k-strided - which runs the forward block projections (on the transposed weights) and the
-    # dgrads: 8 launches per layer, 96 per step, the same four shapes in both directions.
+    # dominant MFMA kernel: gemm64_kernel<128,192,true,true,EpilogueBf16> - both operands contiguous along the
+    # reduced dimension - which runs the forward block projections (on the weights) and the dgrads (on their
+    # transposed copies): 8 launches per layer, 96 per step, the same four shapes in both directions.
     fwd_ms, fwd_launches = profile["gemm_fwd"]
     dgrad_ms, dgrad_launches = profile["gemm_dgrad"]
     launch_ms = (fwd_ms + dgrad_ms) / (fwd_launches + dgrad_launches)
@@ -283,7 +284,7 @@ def main():
                                "wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
                    "global_batch": B, "seq_len": T, "parameters": params, "parallelism": "single GPU"},
         "roofline": {"bound": "mfma",
-                     "kernel": "gemm_kernel<128,192,3,true,false,EpilogueBf16> (forward block projections and "
+                     "kernel": "gemm64_kernel<128,192,true,true,EpilogueBf16> (forward block projections and "
                                "dgrads: QKV, attention-out, MLP-up, MLP-down)",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": HBM_TRAFFIC_PER_LAUNCH,

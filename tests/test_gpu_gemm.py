@@ -105,6 +105,17 @@ def test_dgrad_and_fused_gelu_backward(orc, M, N, K):
                              u.data_ptr(), K))
     sync()
     assert rel(host(dx), orc.gelu_bwd(uh, want)) < 1e-2
+    # the same two products from the transposed weight (Wt[K][N]): same values, same summation order
+    wt = w.t().contiguous()
+    dxt = torch.empty_like(dx)
+    check(lib.tgk_gemm_dgrad_t(stream(), M, N, K, dy.data_ptr(), N, wt.data_ptr(), N, dxt.data_ptr(), K,
+                               u.data_ptr(), K))
+    sync()
+    assert torch.equal(dxt, dx)
+    check(lib.tgk_gemm_dgrad_t(stream(), M, N, K, dy.data_ptr(), N, wt.data_ptr(), N, dxt.data_ptr(), K, None, 0))
+    sync()
+    assert rel(host(dxt), want) < 1e-2
+    assert np.mean(host(dxt) == orc.gemm_dgrad(dyh, wh, emulate=True)) > 0.99
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 128, 128), (256, 256, 192), (1024, 384, 256), (4096, 256, 128),
@@ -179,6 +190,11 @@ def test_full_size_sweep_rows_sampled(orc, N, K):
     check(lib.tgk_gemm_dgrad(stream(), M, N, K, dy.data_ptr(), N, w.data_ptr(), K, dx.data_ptr(), K, None, 0))
     sync()
     assert rel(host(dx)[rows], orc.gemm_dgrad(dyh[rows], wh)) < 1e-2
+    dxt = torch.empty_like(dx)
+    wt = w.t().contiguous()
+    check(lib.tgk_gemm_dgrad_t(stream(), M, N, K, dy.data_ptr(), N, wt.data_ptr(), N, dxt.data_ptr(), K, None, 0))
+    sync()
+    assert torch.equal(dxt, dx)  # the engine's path: 64-k stages on the transposed weight
     need = lib.tgk_gemm_wgrad_workspace(M, N, K)
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
     dw = torch.empty(N, K, dtype=torch.float32, device="cuda")
