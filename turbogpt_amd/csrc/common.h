@@ -24,8 +24,12 @@ TG_DEVICE float bf16_to_float(bf16_t b) {
 TG_DEVICE bf16_t float_to_bf16(float f) {
     return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
+// both halves in one v_cvt_pk_bf16_f32
 TG_DEVICE uint32_t pack_bf16(float lo, float hi) {
-    return uint32_t(float_to_bf16(lo)) | (uint32_t(float_to_bf16(hi)) << 16);
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const f32x2 pair = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
 }
 TG_DEVICE float bf16_lo(uint32_t pair) {
     return __uint_as_float(pair << 16);
@@ -39,28 +43,32 @@ TG_DEVICE float round_bf16(float f) {
 // GELU with the exact-erf definition and its derivative.  erf is evaluated with Abramowitz-Stegun
 // 7.1.26 (|error| <= 1.5e-7, far below bf16 resolution): one reciprocal, one exp2 and a degree-5
 // Horner chain, branch free.  gelu'(x) = Phi(x) + x phi(x) shares the exponential, because
-// erf(x/sqrt2) needs exp(-x^2/2) and so does phi.
+// erf(x/sqrt2) needs exp(-x^2/2) and so does phi.  Constants are folded so that one element costs 13
+// instructions forward: the epilogues that call this are bound by their instruction count.
 struct GeluParts {
-    float cdf; // Phi(x) = 0.5 (1 + erf(x / sqrt 2))
-    float pdf; // phi(x) = exp(-x^2 / 2) / sqrt(2 pi)
+    float tail; // 0.5 erfc(|x| / sqrt 2) = Phi(-|x|)
+    float e;    // exp(-x^2 / 2)
 };
 TG_DEVICE GeluParts gelu_parts(float x) {
-    const float z = fabsf(x) * 0.70710678118654752f;
-    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
-    const float e = __builtin_amdgcn_exp2f(x * x * -0.72134752044448170f); // exp(-x^2/2)
-    float poly = fmaf(1.061405429f, t, -1.453152027f);
-    poly = fmaf(poly, t, 1.421413741f);
-    poly = fmaf(poly, t, -0.284496736f);
-    poly = fmaf(poly, t, 0.254829592f);
-    const float tail = 0.5f * poly * t * e; // 0.5 erfc(|x|/sqrt2)
-    return {x < 0.f ? tail : 1.0f - tail, 0.39894228040143268f * e};
+    const float t = __builtin_amdgcn_rcpf(fmaf(fabsf(x), 0.3275911f * 0.70710678118654752f, 1.0f));
+    const float s = x * 0.84932180028801905f; // s^2 = x^2 / (2 ln 2)
+    const float e = __builtin_amdgcn_exp2f(-(s * s));
+    float poly = fmaf(0.5f * 1.061405429f, t, 0.5f * -1.453152027f);
+    poly = fmaf(poly, t, 0.5f * 1.421413741f);
+    poly = fmaf(poly, t, 0.5f * -0.284496736f);
+    poly = fmaf(poly, t, 0.5f * 0.254829592f);
+    return {poly * t * e, e};
 }
 TG_DEVICE float gelu_f(float x) {
-    return x * gelu_parts(x).cdf;
+    // x Phi(x) = max(x, 0) - |x| Phi(-|x|)
+    float positive; // fmaxf would add a canonicalising v_max x, x in front
+    asm("v_max_f32 %0, 0, %1" : "=v"(positive) : "v"(x));
+    return fmaf(-fabsf(x), gelu_parts(x).tail, positive);
 }
 TG_DEVICE float gelu_grad_f(float x) {
     const GeluParts g = gelu_parts(x);
-    return fmaf(x, g.pdf, g.cdf);
+    const float cdf = x < 0.f ? g.tail : 1.0f - g.tail;
+    return fmaf(x * g.e, 0.39894228040143268f, cdf);
 }
 TG_DEVICE float wave_sum(float x) {
 #pragma unroll
