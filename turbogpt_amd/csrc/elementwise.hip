@@ -24,13 +24,15 @@ TG_DEVICE u32x4 pack8(const float (&f)[8]) {
     return v;
 }
 // fp32 master values of 8 consecutive parameters from their (hi, lo) halves (cuda/ops.cuh:6-9)
-TG_DEVICE void join8(const uint16_t *hi, const uint16_t *lo, float (&f)[8]) {
-    const u32x4 h = *reinterpret_cast<const u32x4 *>(hi), l = *reinterpret_cast<const u32x4 *>(lo);
+TG_DEVICE void join8(const u32x4 &h, const u32x4 &l, float (&f)[8]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         f[2 * i] = __uint_as_float((h[i] << 16) | (l[i] & 0xffffu));
         f[2 * i + 1] = __uint_as_float((h[i] & 0xffff0000u) | (l[i] >> 16));
     }
+}
+TG_DEVICE void join8(const uint16_t *hi, const uint16_t *lo, float (&f)[8]) {
+    join8(*reinterpret_cast<const u32x4 *>(hi), *reinterpret_cast<const u32x4 *>(lo), f);
 }
 TG_DEVICE uint64_t hash_u64(uint64_t x) { // utils.h:13-18
     x += 0x9e3779b97f4a7c15ULL;
@@ -121,10 +123,29 @@ __global__ __launch_bounds__(256) void embed_bwd_positions_kernel(const bf16_t *
 // A row lives in the registers of GROUP lanes (two-pass mean / variance), NC 16-byte chunks per lane
 // (D <= NC * GROUP * 8).  GROUP = 64: one row per wave.  GROUP = 32: two rows per wave, which fits
 // D = 768 (96 chunks = 32 x 3) without idle lane slots and keeps three loads per array in flight.
+// Sum over the GROUP lanes of a row, result in every lane: four DPP steps inside a row of 16 lanes, then the
+// gfx950 lane-swap instructions across rows - all on the vector ALU, no LDS round trips (ds_bpermute, which
+// __shfl_xor compiles to, costs an LDS latency per step and these sums sit on every row's critical path).
+TG_DEVICE float dpp_add(float x, int control) {
+    // control: 0xB1 quad_perm [1,0,3,2], 0x4E quad_perm [2,3,0,1], 0x141 row_half_mirror, 0x140 row_mirror
+    switch (control) {
+    case 0xB1: return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));
+    case 0x4E: return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));
+    case 0x141: return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));
+    default: return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, true));
+    }
+}
 template <int GROUP> TG_DEVICE float group_sum(float x) {
-#pragma unroll
-    for (int k = GROUP / 2; k; k >>= 1)
-        x += __shfl_xor(x, k, 64);
+    x = dpp_add(x, 0xB1);
+    x = dpp_add(x, 0x4E);
+    x = dpp_add(x, 0x141);
+    x = dpp_add(x, 0x140); // every lane of a 16-lane row holds the row's sum
+    const auto rows = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(rows[0]) + __uint_as_float(rows[1]); // rows 0+1 and 2+3
+    if (GROUP == 64) {
+        const auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+        x = __uint_as_float(halves[0]) + __uint_as_float(halves[1]);
+    }
     return x;
 }
 template <int NC, int GROUP>
@@ -138,10 +159,38 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
     constexpr int PER_BLOCK = 256 / GROUP; // rows a block works on at a time
     const int lane = threadIdx.x & (GROUP - 1), slot = threadIdx.x / GROUP, chunks = D >> 3;
     const float inv_d = 1.0f / D;
-    // the row loop is uniform over the wave: a wave's second half may run one row past the end
-    for (int row0 = blockIdx.x * PER_BLOCK; row0 < rows; row0 += gridDim.x * PER_BLOCK) {
+    // gamma and beta are fetched once, ahead of the first row, and stay packed until they are used: behind
+    // the row's reductions they would add a second memory latency to every row
+    u32x4 g_hi[NC], g_lo[NC], b_hi[NC], b_lo[NC];
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+        const int c = lane + j * GROUP;
+        if (c < chunks) {
+            g_hi[j] = *reinterpret_cast<const u32x4 *>(gamma_hi + c * 8);
+            g_lo[j] = *reinterpret_cast<const u32x4 *>(gamma_lo + c * 8);
+            b_hi[j] = *reinterpret_cast<const u32x4 *>(beta_hi + c * 8);
+            b_lo[j] = *reinterpret_cast<const u32x4 *>(beta_lo + c * 8);
+        }
+    }
+    // the row loop is uniform over the wave: a wave's second half may run one row past the end.  The next
+    // row's chunks are requested before the current row is reduced.
+    const int stride = gridDim.x * PER_BLOCK;
+    u32x4 raw[NC];
+    auto fetch = [&](int row, u32x4 (&into)[NC]) {
+#pragma unroll
+        for (int j = 0; j < NC; ++j) {
+            const int c = lane + j * GROUP;
+            into[j] = u32x4{0, 0, 0, 0};
+            if (row < rows && c < chunks)
+                into[j] = *reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8);
+        }
+    };
+    fetch(blockIdx.x * PER_BLOCK + slot, raw);
+    for (int row0 = blockIdx.x * PER_BLOCK; row0 < rows; row0 += stride) {
         const int row = row0 + slot;
         const bool live = row < rows;
+        u32x4 next[NC];
+        fetch(row0 + stride < rows ? row + stride : rows, next);
         float v[NC][8];
         float sum = 0.f;
 #pragma unroll
@@ -151,11 +200,12 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
             for (int k = 0; k < 8; ++k)
                 v[j][k] = 0.f;
             if (live && c < chunks) {
-                unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
+                unpack8(raw[j], v[j]);
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
                     sum += v[j][k];
             }
+            raw[j] = next[j];
         }
         const float mean = group_sum<GROUP>(sum) * inv_d;
         float sq = 0.f;
@@ -173,8 +223,8 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(const bf16_t *__rest
             const int c = lane + j * GROUP;
             if (live && c < chunks) {
                 float gm[8], bt[8], o[8];
-                join8(gamma_hi + c * 8, gamma_lo + c * 8, gm);
-                join8(beta_hi + c * 8, beta_lo + c * 8, bt);
+                join8(g_hi[j], g_lo[j], gm);
+                join8(b_hi[j], b_lo[j], bt);
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
                     o[k] = v[j][k] * inv * gm[k] + bt[k];
@@ -210,17 +260,25 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
     for (int row0 = blockIdx.x * PER_BLOCK; row0 < rows; row0 += gridDim.x * PER_BLOCK) {
         const int row = row0 + slot;
         const bool live = row < rows;
+        // the row's residual gradient is only needed at the end, but requested with x and dy: behind the
+        // reductions it would add a second memory latency to every row
+        u32x4 prior_raw[NC];
         float v[NC][8], g[NC][8];
         float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < NC; ++j) {
             const int c = lane + j * GROUP;
+            prior_raw[j] = u32x4{0, 0, 0, 0};
 #pragma unroll
             for (int k = 0; k < 8; ++k)
                 v[j][k] = g[j][k] = 0.f;
             if (live && c < chunks) {
-                unpack8(*reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8), v[j]);
-                unpack8(*reinterpret_cast<const u32x4 *>(dy + size_t(row) * D + c * 8), g[j]);
+                const u32x4 rx = *reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8);
+                const u32x4 rg = *reinterpret_cast<const u32x4 *>(dy + size_t(row) * D + c * 8);
+                if (residual)
+                    prior_raw[j] = *reinterpret_cast<const u32x4 *>(dx + size_t(row) * D + c * 8);
+                unpack8(rx, v[j]);
+                unpack8(rg, g[j]);
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
                     sum += v[j][k];
@@ -264,7 +322,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
                 if (residual) {
                     // residual gradients stay in bf16 between operators (cuda/ops.cuh:74-76)
                     float prior[8];
-                    unpack8(*reinterpret_cast<const u32x4 *>(p), prior);
+                    unpack8(prior_raw[j], prior);
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
                         o[k] = prior[k] + round_bf16(o[k]);
@@ -636,7 +694,9 @@ extern "C" int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint
         aligned(beta_hi, "layernorm: beta_hi");
         aligned(beta_lo, "layernorm: beta_lo");
         const LayerNormShape shape = layernorm_shape(D);
-        const dim3 grid(grid_for(rows, 256 / shape.group, 8192));
+        // two blocks per CU (256 CUs), each walking its rows with gamma and beta in registers: measured best
+        // of 256..2048 blocks at 16384 rows
+        const dim3 grid(grid_for(rows, 256 / shape.group, 512));
 #define TG_LN_FWD(NC, GROUP)                                                                                      \
     hipLaunchKernelGGL((layernorm_fwd_kernel<NC, GROUP>), grid, dim3(256), 0, stream, x, gamma_hi, gamma_lo,      \
                        beta_hi, beta_lo, y, rows, D, eps)
@@ -656,7 +716,7 @@ extern "C" int tgk_layernorm_fwd(hipStream_t stream, int rows, int D, const uint
 }
 
 static int layernorm_bwd_blocks(int rows) {
-    return grid_for(rows, 8, 1024);
+    return grid_for(rows, 8, 768); // three blocks per CU: measured best of 512 / 768 / 1024 at 16384 rows
 }
 extern "C" size_t tgk_layernorm_bwd_workspace(int rows, int D) {
     return rows > 0 && D > 0 ? size_t(layernorm_bwd_blocks(rows)) * 2 * D * sizeof(float) : 0;
