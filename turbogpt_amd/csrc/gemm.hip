@@ -92,9 +92,18 @@ struct EpilogueF32 {
 // bf16 outputs: each 32x32 accumulator tile is rounded and transposed through a wave-private LDS buffer
 // (32 rows of 64 bytes, 16-byte chunk c of row r at c ^ ((r >> 2) & 3)), so that a lane finishes 8
 // consecutive n of rows get_row and get_row + 16.  LDS operations of one wave execute in order, so no
-// barrier is needed around the buffer.
-template <int FM, int FN, class Epilogue, class Aux>
-TG_DEVICE void staged_store_bf16(const f32x16 (&acc)[FM][FN], const Aux &aux, unsigned char *mine,
+// barrier is needed around the buffer.  The epilogue's second input (residual, saved pre-activation) is
+// fetched in that row layout one 32x32 tile ahead; `first` is the pair for tile (0, 0), requested by the
+// caller before its last MFMAs (load_aux_pair) - holding all FM x FN pairs there costs 48 registers.
+template <int FM, int FN, class Epilogue>
+TG_DEVICE void load_aux_pair(const Epilogue &epilogue, int tile, int m_base, int n_base, int lane, u32x4 (&pair)[2]) {
+    const int i = tile / FN, j = tile - i * FN;
+    const int m = m_base + i * 32 + (lane >> 2), n = n_base + j * 32 + (lane & 3) * 8;
+    pair[0] = epilogue.load_aux(m, n);
+    pair[1] = epilogue.load_aux(m + 16, n);
+}
+template <int FM, int FN, class Epilogue>
+TG_DEVICE void staged_store_bf16(const f32x16 (&acc)[FM][FN], const u32x4 (&first)[2], unsigned char *mine,
                                  const Epilogue &epilogue, int m_base, int n_base, int lane) {
     const int get_row = lane >> 2, get_chunk = lane & 3;
     const int row = lane & 31;
@@ -102,10 +111,15 @@ TG_DEVICE void staged_store_bf16(const f32x16 (&acc)[FM][FN], const Aux &aux, un
     const int put_swizzle = (row >> 2) & 3;
     // rows r and r + 16 share a swizzle term, so the second half is 1 KiB further on
     const unsigned char *get = mine + get_row * 64 + ((get_chunk ^ ((get_row >> 2) & 3)) << 4);
+    const bool wants_aux = epilogue.wants_aux();
+    u32x4 aux[2] = {first[0], first[1]};
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
+            u32x4 next[2] = {aux[0], aux[1]};
+            if (wants_aux && i * FN + j + 1 < FM * FN)
+                load_aux_pair<FM, FN>(epilogue, i * FN + j + 1, m_base, n_base, lane, next);
             const int m = m_base + i * 32 + get_row, n = n_base + j * 32 + get_chunk * 8;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -114,8 +128,10 @@ TG_DEVICE void staged_store_bf16(const f32x16 (&acc)[FM][FN], const Aux &aux, un
                 packed.y = pack_bf16(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
                 *reinterpret_cast<u32x2 *>(put + ((q ^ put_swizzle) << 4)) = packed;
             }
-            epilogue.finish(m, n, *reinterpret_cast<const u32x4 *>(get), aux[i][j][0]);
-            epilogue.finish(m + 16, n, *reinterpret_cast<const u32x4 *>(get + 1024), aux[i][j][1]);
+            epilogue.finish(m, n, *reinterpret_cast<const u32x4 *>(get), aux[0]);
+            epilogue.finish(m + 16, n, *reinterpret_cast<const u32x4 *>(get + 1024), aux[1]);
+            aux[0] = next[0];
+            aux[1] = next[1];
         }
 }
 
@@ -353,21 +369,12 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(const bf16_t *__restrict__
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     acc[i][j][r] = 0.f;
-        // row layout of the staged epilogue: this lane finishes rows get_row and get_row + 16, 8 columns
-        const int get_row = lane >> 2, get_chunk = lane & 3;
-        u32x4 aux[Epilogue::BF16 ? FM : 1][Epilogue::BF16 ? FN : 1][2];
+        u32x4 aux[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}}; // the epilogue's second input for tile (0, 0)
         const int aux_at = nk > 2 ? nk - 2 : 0;
         for (int kt = 0; kt < nk; ++kt) {
-            if (Epilogue::BF16 && kt == aux_at && epilogue.wants_aux()) {
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-#pragma unroll
-                        for (int half = 0; half < 2; ++half)
-                            aux[Epilogue::BF16 ? i : 0][Epilogue::BF16 ? j : 0][half] = epilogue.load_aux(
-                                m0 + wm + i * 32 + get_row + half * 16, n0 + wn + j * 32 + get_chunk * 8);
-            }
+            if constexpr (Epilogue::BF16)
+                if (kt == aux_at && epilogue.wants_aux())
+                    load_aux_pair<FM, FN>(epilogue, 0, m0 + wm, n0 + wn, lane, aux);
             // in flight now: the stage being consumed (landed), then inflight-1 younger ones; the next one
             // must land too
             wait_stages(inflight >= 2 ? inflight - 2 : 0);
@@ -539,22 +546,13 @@ __global__ __launch_bounds__(256, 2) void gemm64_kernel(const bf16_t *__restrict
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     acc[i][j][r] = 0.f;
-        const int get_row = lane >> 2, get_chunk = lane & 3;
-        u32x4 aux[Epilogue::BF16 ? FM : 1][Epilogue::BF16 ? FN : 1][2];
+        u32x4 aux[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}}; // the epilogue's second input for tile (0, 0)
         for (int c = 0; c < nc; ++c) {
             wait_vmcnt<0>(); // this wave's copies of stage c (and the previous tile's stores) are done
             __syncthreads(); // everyone's are, and everyone is done reading the other slot
-            if (Epilogue::BF16 && c == nc - 1 && epilogue.wants_aux()) {
-                // the epilogue's second input, in its row layout, lands while the last stage is multiplied
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-#pragma unroll
-                        for (int half = 0; half < 2; ++half)
-                            aux[Epilogue::BF16 ? i : 0][Epilogue::BF16 ? j : 0][half] = epilogue.load_aux(
-                                m0 + wm + i * 32 + get_row + half * 16, n0 + wn + j * 32 + get_chunk * 8);
-            }
+            if constexpr (Epilogue::BF16)
+                if (c == nc - 1 && epilogue.wants_aux())
+                    load_aux_pair<FM, FN>(epilogue, 0, m0 + wm, n0 + wn, lane, aux); // lands during the last stage
             bool copy = true;
             if (p_left == 0) {
                 p_item += stride;
