@@ -74,6 +74,26 @@ TGK_API int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uint16
                    size_t workspace_bytes);
 TGK_API size_t tgk_gemm_wgrad_workspace(int M, int N, int K);
 
+/* Up to four weight gradients that share the reduced dimension M (the tokens) in one launch, e.g. the four of
+ * a transformer block: dW_j[N_j][K_j] (= | +=) dY_j[M][N_j]^T . X_j[M][K_j], fp32, deterministic.  The output
+ * tiles of all jobs are cut into equal runs of work over the resident blocks, so the matrices need not fill the
+ * GPU one by one and far fewer partial sums are written than by one tgk_gemm_wgrad per matrix.  Every N_j a
+ * multiple of 128, every K_j of 192, M of 64.  `workspace` holds tgk_gemm_wgrad_batch_workspace(M, count, jobs)
+ * bytes.  No counterpart in the reference, which computes one weight_gradient at a time (cuda/ops.cuh:83-109). */
+typedef struct TgkWgradJob {
+    int N, K;
+    const uint16_t *dY;
+    int lddy;
+    const uint16_t *X;
+    int ldx;
+    float *dW;
+    int lddw;
+} TgkWgradJob;
+TGK_API int tgk_gemm_wgrad_batch(hipStream_t stream, int M, int count, const TgkWgradJob *jobs, int accumulate,
+                                 void *workspace, size_t workspace_bytes);
+TGK_API size_t tgk_gemm_wgrad_batch_workspace(int M, int count, const TgkWgradJob *jobs);
+
+
 /* ---- Causal softmax attention, head_dim 64.  Takes the slot of attention_forward /
  * attention_backward (cuda/attention.cuh:48-106); the reference's arg-max attention is replaced
  * by softmax(Q K^T * scale + causal mask) V as the target specifies.  Layout is the reference's
@@ -121,6 +141,12 @@ TGK_API int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint16_
                               const uint16_t *gamma_hi, const uint16_t *gamma_lo, uint16_t *dx,
                               float *dgamma, float *dbeta, float eps, int residual, int accumulate,
                               void *workspace, size_t workspace_bytes);
+/* The same with the residual gradient taken from a buffer of its own: dx = RN_bf16(residual + RN_bf16(LN'(x) dy));
+ * residual may be NULL (no addition) or dx itself.  Lets a caller keep the incoming gradient for later use. */
+TGK_API int tgk_layernorm_bwd_add(hipStream_t stream, int rows, int D, const uint16_t *x, const uint16_t *dy,
+                                  const uint16_t *gamma_hi, const uint16_t *gamma_lo, const uint16_t *residual,
+                                  uint16_t *dx, float *dgamma, float *dbeta, float eps, int accumulate,
+                                  void *workspace, size_t workspace_bytes);
 TGK_API size_t tgk_layernorm_bwd_workspace(int rows, int D);
 
 /* Softmax cross-entropy over 256 byte classes on bf16 logits [rows][256] (cuda/model.cuh:33-58):

@@ -145,6 +145,89 @@ def test_wgrad_split_k_and_accumulate(orc, M, N, K):
     np.testing.assert_array_equal(host(dw2), first)
 
 
+def run_wgrad_batch(M, shapes, rng, accumulate=0, start=0.0):
+    """One tgk_gemm_wgrad_batch over `shapes` (N, K); returns (gradients, inputs)."""
+    import ctypes as C
+    from turbogpt_amd.bridge import WgradJob
+    lib = library()
+    jobs = (WgradJob * len(shapes))()
+    keep, inputs = [], []
+    for j, (N, K) in enumerate(shapes):
+        dy, dyh = to_bf16_device(rng.standard_normal((M, N)))
+        x, xh = to_bf16_device(rng.standard_normal((M, K)))
+        dw = torch.full((N, K), start, dtype=torch.float32, device="cuda")
+        keep.append((dy, x, dw))
+        inputs.append((dyh, xh))
+        jobs[j] = WgradJob(N, K, dy.data_ptr(), N, x.data_ptr(), K, dw.data_ptr(), K)
+    need = lib.tgk_gemm_wgrad_batch_workspace(M, len(shapes), C.addressof(jobs))
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    check(lib.tgk_gemm_wgrad_batch(stream(), M, len(shapes), C.addressof(jobs), accumulate, ws.data_ptr(), need))
+    sync()
+    return keep, inputs, (jobs, ws, need)
+
+
+@pytest.mark.parametrize("M,shapes", [(64, [(128, 192)]), (256, [(128, 192), (256, 384)]),
+                                      (2048, [(768, 768), (256, 192), (128, 576), (384, 192)]),
+                                      (4096, [(128, 192), (128, 192), (128, 192)])])
+def test_wgrad_batch_against_the_checker(orc, M, shapes):
+    """Several weight gradients in one launch: every job against the checker, accumulate, and a second run
+    bit-identical (runs and pieces are summed in a fixed order)."""
+    lib = library()
+    keep, inputs, (jobs, ws, need) = run_wgrad_batch(M, shapes, np.random.default_rng(M + len(shapes)), start=3.0)
+    firsts = []
+    for (dy, x, dw), (dyh, xh) in zip(keep, inputs):
+        assert rel(host(dw), orc.gemm_wgrad(dyh, xh)) < 1e-4
+        firsts.append(host(dw).copy())
+    import ctypes as C
+    check(lib.tgk_gemm_wgrad_batch(stream(), M, len(shapes), C.addressof(jobs), 1, ws.data_ptr(), need))
+    sync()
+    for (dy, x, dw), first in zip(keep, firsts):
+        np.testing.assert_allclose(host(dw), 2 * first, rtol=1e-6)
+    check(lib.tgk_gemm_wgrad_batch(stream(), M, len(shapes), C.addressof(jobs), 0, ws.data_ptr(), need))
+    sync()
+    for (dy, x, dw), first in zip(keep, firsts):
+        np.testing.assert_array_equal(host(dw), first)
+
+
+def test_wgrad_batch_of_a_block_at_full_size(orc):
+    """The four weight gradients of one transformer block at M = 16384 in one launch, against one
+    tgk_gemm_wgrad per matrix (fp32 sums in a different order: 1e-5) and the checker on sampled rows."""
+    lib = library()
+    M = 16384
+    shapes = [(768, 3072), (3072, 768), (768, 768), (2304, 768)]
+    rng = np.random.default_rng(99)
+    keep, inputs, _ = run_wgrad_batch(M, shapes, rng)
+    for (dy, x, dw), (dyh, xh), (N, K) in zip(keep, inputs, shapes):
+        need = lib.tgk_gemm_wgrad_workspace(M, N, K)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        single = torch.empty(N, K, dtype=torch.float32, device="cuda")
+        check(lib.tgk_gemm_wgrad(stream(), M, N, K, dy.data_ptr(), N, x.data_ptr(), K, single.data_ptr(), K, 0,
+                                 ws.data_ptr(), need))
+        sync()
+        assert rel(host(dw), host(single)) < 1e-5
+        cols = np.sort(rng.choice(N, 24, replace=False))
+        assert rel(host(dw)[cols], orc.gemm_wgrad(np.ascontiguousarray(dyh[:, cols]), xh)) < 1e-4
+
+
+def test_wgrad_batch_rejects_bad_jobs():
+    import ctypes as C
+    from turbogpt_amd.bridge import WgradJob
+    lib = library()
+    t = torch.zeros(256 * 256, dtype=torch.bfloat16, device="cuda")
+    f = torch.zeros(256 * 256, dtype=torch.float32, device="cuda")
+    jobs = (WgradJob * 1)(WgradJob(128, 128, t.data_ptr(), 128, t.data_ptr(), 128, f.data_ptr(), 128))
+    assert lib.tgk_gemm_wgrad_batch_workspace(64, 1, C.addressof(jobs)) == 0
+    assert lib.tgk_gemm_wgrad_batch(stream(), 64, 1, C.addressof(jobs), 0, t.data_ptr(), 1 << 20) == -1
+    assert b"every K of 192" in lib.tgk_error()
+    jobs[0].K = jobs[0].ldx = jobs[0].lddw = 192
+    assert lib.tgk_gemm_wgrad_batch(stream(), 60, 1, C.addressof(jobs), 0, t.data_ptr(), 1 << 20) == -1
+    assert lib.tgk_gemm_wgrad_batch(stream(), 64, 5, C.addressof(jobs), 0, t.data_ptr(), 1 << 20) == -1
+    assert lib.tgk_gemm_wgrad_batch(stream(), 64, 1, C.addressof(jobs), 0, None, 0) == -1
+    assert b"workspace" in lib.tgk_error()
+    sync()
+
+
 def test_strided_views_of_a_packed_buffer(orc):
     # the engine hands out column slices of wider buffers: leading dimensions differ from widths
     lib = library()

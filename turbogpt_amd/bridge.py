@@ -23,6 +23,8 @@ KERNEL_ABI = {
     "tgk_gemm_dgrad_t": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, vp, i32]),
     "tgk_gemm_wgrad": (i32, [vp, i32, i32, i32, vp, i32, vp, i32, vp, i32, i32, vp, sz]),
     "tgk_gemm_wgrad_workspace": (sz, [i32, i32, i32]),
+    "tgk_gemm_wgrad_batch": (i32, [vp, i32, i32, vp, i32, vp, sz]),
+    "tgk_gemm_wgrad_batch_workspace": (sz, [i32, i32, vp]),
     "tgk_attn_fwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, f32]),
     "tgk_attn_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32,
                            f32, vp, sz]),
@@ -32,6 +34,7 @@ KERNEL_ABI = {
     "tgk_embed_bwd_workspace": (sz, [i32, i32]),
     "tgk_layernorm_fwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, f32]),
     "tgk_layernorm_bwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, f32, i32, i32, vp, sz]),
+    "tgk_layernorm_bwd_add": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, f32, i32, vp, sz]),
     "tgk_layernorm_bwd_workspace": (sz, [i32, i32]),
     "tgk_cross_entropy": (i32, [vp, i32, i32, vp, vp, vp, vp, f32, i32]),
     "tgk_sumsq_partials": (i32, [vp, vp, sz, vp, i32]),
@@ -58,6 +61,12 @@ class Config(C.Structure):
         super().__init__(4, 4, 16, 0, 0, 5, .0006, .02, .9, .95, .95, .1, 1e-8, 1., 3407, 1)
         for key, value in kwargs.items():
             setattr(self, key, value)
+
+
+class WgradJob(C.Structure):
+    """TgkWgradJob of include/tgk_kernels.h: one dW[N][K] = dY[M][N]^T X[M][K] of a batch."""
+    _fields_ = [("N", C.c_int), ("K", C.c_int), ("dY", C.c_void_p), ("lddy", C.c_int), ("X", C.c_void_p),
+                ("ldx", C.c_int), ("dW", C.c_void_p), ("lddw", C.c_int)]
 
 
 class ModelConfig(C.Structure):

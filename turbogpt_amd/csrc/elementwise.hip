@@ -240,9 +240,9 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
                                                             const bf16_t *__restrict__ dy,
                                                             const uint16_t *__restrict__ gamma_hi,
                                                             const uint16_t *__restrict__ gamma_lo,
-                                                            bf16_t *__restrict__ dx,
+                                                            const bf16_t *residual, bf16_t *dx,
                                                             float *__restrict__ partial, int rows, int D,
-                                                            float eps, int residual) {
+                                                            float eps) {
     constexpr int PER_BLOCK = 256 / GROUP;
     extern __shared__ float lds[]; // [PER_BLOCK row slots][2][D]
     const int lane = threadIdx.x & (GROUP - 1), slot = threadIdx.x / GROUP, chunks = D >> 3;
@@ -275,8 +275,8 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(const bf16_t *__rest
             if (live && c < chunks) {
                 const u32x4 rx = *reinterpret_cast<const u32x4 *>(x + size_t(row) * D + c * 8);
                 const u32x4 rg = *reinterpret_cast<const u32x4 *>(dy + size_t(row) * D + c * 8);
-                if (residual)
-                    prior_raw[j] = *reinterpret_cast<const u32x4 *>(dx + size_t(row) * D + c * 8);
+                if (residual) // may be dx itself: every lane reads its chunk before it writes it
+                    prior_raw[j] = *reinterpret_cast<const u32x4 *>(residual + size_t(row) * D + c * 8);
                 unpack8(rx, v[j]);
                 unpack8(rg, g[j]);
 #pragma unroll
@@ -721,10 +721,10 @@ static int layernorm_bwd_blocks(int rows) {
 extern "C" size_t tgk_layernorm_bwd_workspace(int rows, int D) {
     return rows > 0 && D > 0 ? size_t(layernorm_bwd_blocks(rows)) * 2 * D * sizeof(float) : 0;
 }
-extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint16_t *x,
-                                 const uint16_t *dy, const uint16_t *gamma_hi, const uint16_t *gamma_lo,
-                                 uint16_t *dx, float *dgamma, float *dbeta, float eps, int residual,
-                                 int accumulate, void *workspace, size_t workspace_bytes) {
+extern "C" int tgk_layernorm_bwd_add(hipStream_t stream, int rows, int D, const uint16_t *x,
+                                     const uint16_t *dy, const uint16_t *gamma_hi, const uint16_t *gamma_lo,
+                                     const uint16_t *residual, uint16_t *dx, float *dgamma, float *dbeta,
+                                     float eps, int accumulate, void *workspace, size_t workspace_bytes) {
     return guarded([&] {
         require(rows > 0 && D > 0 && D % 64 == 0 && D <= MAX_LN_CHUNKS * 512,
                 "layernorm_bwd: D must be a multiple of 64, at most 2048");
@@ -733,6 +733,8 @@ extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint
         aligned(dx, "layernorm: dx");
         aligned(gamma_hi, "layernorm: gamma_hi");
         aligned(gamma_lo, "layernorm: gamma_lo");
+        if (residual)
+            aligned(residual, "layernorm: residual");
         require(dgamma && dbeta, "layernorm_bwd: missing operand");
         require(workspace && workspace_bytes >= tgk_layernorm_bwd_workspace(rows, D),
                 "layernorm_bwd: workspace too small (see tgk_layernorm_bwd_workspace)");
@@ -744,7 +746,7 @@ extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint
         const size_t lds = size_t(4) * 2 * D * sizeof(float);
 #define TG_LN_BWD(NC, GROUP)                                                                                      \
     hipLaunchKernelGGL((layernorm_bwd_kernel<NC, GROUP>), dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,  \
-                       gamma_lo, dx, partial, rows, D, eps, residual)
+                       gamma_lo, residual, dx, partial, rows, D, eps)
         if (per_lane == 1)
             TG_LN_BWD(1, 64);
         else if (per_lane == 2)
@@ -756,6 +758,13 @@ extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint
                            dgamma, dbeta, accumulate);
         check_hip(hipGetLastError(), "layernorm_bwd launch: ");
     });
+}
+extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint16_t *x,
+                                 const uint16_t *dy, const uint16_t *gamma_hi, const uint16_t *gamma_lo,
+                                 uint16_t *dx, float *dgamma, float *dbeta, float eps, int residual,
+                                 int accumulate, void *workspace, size_t workspace_bytes) {
+    return tgk_layernorm_bwd_add(stream, rows, D, x, dy, gamma_hi, gamma_lo, residual ? dx : nullptr, dx, dgamma,
+                                 dbeta, eps, accumulate, workspace, workspace_bytes);
 }
 
 extern "C" int tgk_cross_entropy(hipStream_t stream, int rows, int vocab, uint16_t *logits,

@@ -69,6 +69,7 @@ struct Slot {
     std::vector<bf16_t *> x; // x[l] = input of block l; x[depth] = output of the last block
     std::vector<LayerBuffers> layers;
     bf16_t *nf = nullptr, *logits = nullptr, *dh = nullptr, *t1 = nullptr, *du = nullptr, *dqkv = nullptr;
+    bf16_t *dh_mid = nullptr; // the gradient between a block's two halves, when the block's weight gradients are batched
     void *workspace = nullptr;
 };
 // One immutable copy of the weights: a batch reads a single version from its first kernel to its last
@@ -101,6 +102,7 @@ struct Engine {
     int64_t data_size = 0;
     float *logits_f32 = nullptr;
     size_t workspace_bytes = 0;
+    bool batched_wgrad = false; // a block's four weight gradients in one launch (shapes permitting)
 
     std::vector<StepRates> schedule;
     uint64_t step = 0;
@@ -275,6 +277,31 @@ struct Engine {
         for (int l = c.depth - 1; l >= 0; --l) {
             const TgLayerParameters &p = layout.layers[l];
             LayerBuffers &b = layers[l];
+            if (batched_wgrad) {
+                // The four weight gradients wait until all their operands exist (after the attention backward) and
+                // go out as one launch; for that the gradient entering the block (dh) survives the block's first
+                // half: LayerNorm 2 writes its sum with dh into dh_mid.
+                bf16_t *mid = s.dh_mid;
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, du, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
+                OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_add(stream, M, d, b.mid, t1, w(p.ln2_g), wl(p.ln2_g), dh, mid,
+                                                                 g + p.ln2_g, g + p.ln2_b, config.ln_eps, 0, workspace,
+                                                                 workspace_bytes));
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, d, mid, d, wt(p.attn_out), d, t1, d, nullptr, 0));
+                OP(TG_CLASS_ATTN_BWD, tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d,
+                                                   b.qkv + 2 * d, 3 * d, b.o, d, b.lse, t1, d, dqkv, dqkv + d, dqkv + 2 * d,
+                                                   3 * d, scale, workspace, workspace_bytes));
+                const TgkWgradJob jobs[4] = {{d, F, dh, d, b.a, F, g + p.mlp_down, F},
+                                             {F, d, du, F, b.n2, d, g + p.mlp_up, d},
+                                             {d, d, mid, d, b.o, d, g + p.attn_out, d},
+                                             {3 * d, d, dqkv, 3 * d, b.n1, d, g + p.qkv, d}};
+                OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad_batch(stream, M, 4, jobs, 0, workspace, workspace_bytes));
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, 3 * d, d, dqkv, 3 * d, wt(p.qkv), 3 * d, t1, d, nullptr, 0));
+                OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_add(stream, M, d, x[l], t1, w(p.ln1_g), wl(p.ln1_g), mid, dh,
+                                                                 g + p.ln1_g, g + p.ln1_b, config.ln_eps, 0, workspace,
+                                                                 workspace_bytes));
+                continue;
+            }
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, F, dh, d, b.a, F, g + p.mlp_down, F, 0, workspace, workspace_bytes));
             OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, F, d, du, F, b.n2, d, g + p.mlp_up, d, 0, workspace, workspace_bytes));
@@ -627,7 +654,16 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
             e->allocate(slot.du, M * F, false);
             e->allocate(slot.dqkv, M * 3 * d, false);
         }
-        size_t need = tgk_attn_bwd_workspace(c.batch, model->heads, c.context);
+        const TgkWgradJob block_jobs[4] = {{int(d), int(F), nullptr, int(d), nullptr, int(F), nullptr, int(F)},
+                                           {int(F), int(d), nullptr, int(F), nullptr, int(d), nullptr, int(d)},
+                                           {int(d), int(d), nullptr, int(d), nullptr, int(d), nullptr, int(d)},
+                                           {int(3 * d), int(d), nullptr, int(3 * d), nullptr, int(d), nullptr, int(d)}};
+        const size_t batch_need = tgk_gemm_wgrad_batch_workspace(int(M), 4, block_jobs);
+        e->batched_wgrad = batch_need > 0;
+        if (e->batched_wgrad)
+            for (Slot &slot : e->slots)
+                e->allocate(slot.dh_mid, M * d, false);
+        size_t need = std::max(batch_need, tgk_attn_bwd_workspace(c.batch, model->heads, c.context));
         need = std::max(need, tgk_layernorm_bwd_workspace(int(M), int(d)));
         need = std::max(need, tgk_embed_bwd_workspace(int(M), int(d)));
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(V), int(d)));

@@ -449,6 +449,45 @@ template <int ROWS, bool KC> struct Tile64Of;
 template <int ROWS> struct Tile64Of<ROWS, true> { using type = TileKC64<ROWS>; };
 template <int ROWS> struct Tile64Of<ROWS, false> { using type = TileKS64<ROWS>; };
 
+// One 64-k stage of a wave's FM x FN tiles: fragments of the next 16-k step are read while the current MFMAs
+// run, and copy number n of the next stage goes out behind MFMA 2n + 1 (see gemm64_kernel).
+template <class TA, class TB, int FM, int FN, int LOADS, class Copy>
+TG_DEVICE void multiply_stage(f32x16 (&acc)[FM][FN], const unsigned char *slot, int wm, int wn, int lane, bool copy,
+                              Copy &&copy_one) {
+    const unsigned char *sa = slot, *sb = sa + TA::BYTES;
+    bf16x8 af[2][FM], bfr[2][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+        af[0][i] = TA::frag(sa, wm + i * 32, 0, lane);
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+        bfr[0][j] = TB::frag(sb, wn + j * 32, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        if (ks < 3) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                af[(ks + 1) & 1][i] = TA::frag(sa, wm + i * 32, ks + 1, lane);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                bfr[(ks + 1) & 1][j] = TB::frag(sb, wn + j * 32, ks + 1, lane);
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ks & 1][j], af[ks & 1][i], acc[i][j], 0, 0, 0);
+                const int q = ks * FM * FN + i * FN + j; // MFMA number within the stage
+                if ((q & 1) && (q >> 1) < LOADS) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (copy)
+                        copy_one(q >> 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+    }
+}
+
 // The same product as gemm_kernel with two 64-k stages of (BM + BN) * 128 bytes: per stage one wait, one barrier,
 // and the copies of the next stage issued one behind every second MFMA.  A copy instruction that finds the
 // vector-memory queue full stalls its wave, and with it the wave's MFMAs; kept apart, the copies overlap them
@@ -560,38 +599,7 @@ __global__ __launch_bounds__(256, 2) void gemm64_kernel(const bf16_t *__restrict
                 if (copy)
                     producer_open();
             }
-            const unsigned char *sa = smem + c_slot * SLOT, *sb = sa + TA::BYTES;
-            bf16x8 af[2][FM], bfr[2][FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-                af[0][i] = TA::frag(sa, wm + i * 32, 0, lane);
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-                bfr[0][j] = TB::frag(sb, wn + j * 32, 0, lane);
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                if (ks < 3) {
-#pragma unroll
-                    for (int i = 0; i < FM; ++i)
-                        af[(ks + 1) & 1][i] = TA::frag(sa, wm + i * 32, ks + 1, lane);
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        bfr[(ks + 1) & 1][j] = TB::frag(sb, wn + j * 32, ks + 1, lane);
-                }
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int j = 0; j < FN; ++j) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ks & 1][j], af[ks & 1][i], acc[i][j], 0, 0, 0);
-                        const int q = ks * FM * FN + i * FN + j; // MFMA number within the stage
-                        if ((q & 1) && (q >> 1) < LOADS) {
-                            __builtin_amdgcn_sched_barrier(0);
-                            if (copy)
-                                copy_one(q >> 1);
-                            __builtin_amdgcn_sched_barrier(0);
-                        }
-                    }
-            }
+            multiply_stage<TA, TB, FM, FN, LOADS>(acc, smem + c_slot * SLOT, wm, wn, lane, copy, copy_one);
             if (copy) {
                 --p_left;
                 p_slot ^= 1;
@@ -608,6 +616,186 @@ __global__ __launch_bounds__(256, 2) void gemm64_kernel(const bf16_t *__restrict
             staged_store_f32<FM, FN>(acc, slot + wave * 4096, epilogue, m0 + wm, n0 + wn, lane, split);
     }
     wait_vmcnt<0>();
+}
+
+// ---- several weight gradients in one launch ------------------------------------------------------
+// dW_j[N_j][K_j] = dY_j^T X_j for up to four (dY, X) pairs that share the reduced dimension (the tokens).  One
+// matrix rarely has as many 128x192 tiles as the GPU holds blocks, and split into as many token ranges as fill
+// it, it writes that many fp32 partial sums per tile.  Here the tiles of all jobs form one list, cut in two
+// groups: the first `tiles_a` tiles are split `splits_a` ways and the rest `splits_b` ways, chosen so that
+// each group makes one work item per resident block and every block gets one long and one short item of the
+// same total length (four gradients of a d = 768 block: 256 tiles x 2 + 32 tiles x 16 on 512 blocks, 144
+// chunks of 64 tokens each, 98 MB of partial sums instead of 193 MB, one prologue and one tail instead of
+// four).  Within a group the blocks of an XCD work on the same token range of neighbouring tiles, so the rows
+// of dY^T and X they share are read from HBM once per XCD.  wgrad_batch_fold_kernel sums a tile's pieces in
+// split order (fixed, bit-reproducible); a tile that is not split writes the gradient itself.
+constexpr int MAX_WGRAD_JOBS = 4;
+struct WgradBatch {
+    const bf16_t *dy[MAX_WGRAD_JOBS], *x[MAX_WGRAD_JOBS];
+    float *dw[MAX_WGRAD_JOBS];
+    int lddy[MAX_WGRAD_JOBS], ldx[MAX_WGRAD_JOBS], lddw[MAX_WGRAD_JOBS];
+    int tiles_n[MAX_WGRAD_JOBS];
+    int first_tile[MAX_WGRAD_JOBS + 1]; // tiles before job j; [count] = all tiles
+    int count;
+    int k_chunks;            // tokens / 64
+    int tiles_a, splits_a;   // group a: tiles [0, tiles_a)
+    int tiles_b, splits_b;   // group b: the rest
+    int accumulate;
+    float *pieces; // BM * BN floats per (tile, split), tile-local row-major, see piece_slot()
+};
+struct WgradTile {
+    int job, m0, n0;
+};
+struct WgradItem {
+    int tile, split, splits, c0, nc;
+};
+template <int BM, int BN> TG_DEVICE WgradTile wgrad_tile(const WgradBatch &w, int tile) {
+    int job = 0;
+#pragma unroll
+    for (int j = 1; j < MAX_WGRAD_JOBS; ++j)
+        if (j < w.count && tile >= w.first_tile[j])
+            job = j;
+    const int local = tile - w.first_tile[job];
+    return {job, (local / w.tiles_n[job]) * BM, (local % w.tiles_n[job]) * BN};
+}
+TG_DEVICE int piece_slot(const WgradBatch &w, int tile, int split) {
+    return (tile < w.tiles_a ? tile * w.splits_a : w.tiles_a * w.splits_a + (tile - w.tiles_a) * w.splits_b) + split;
+}
+// The block's item of group `group` (0: a, 1: b); false when the group has no item for it.  Consecutive block
+// ids sit on consecutive XCDs; an XCD owns a contiguous range of (split, tile), split-major.
+TG_DEVICE bool wgrad_item(const WgradBatch &w, int group, int block, WgradItem &item) {
+    const int tiles = group ? w.tiles_b : w.tiles_a, splits = group ? w.splits_b : w.splits_a;
+    const int n = tiles * splits;
+    if (block >= n)
+        return false;
+    const int logical = (n & 7) == 0 ? (block & 7) * (n >> 3) + (block >> 3) : block;
+    item.split = logical / tiles;
+    item.tile = (group ? w.tiles_a : 0) + logical - item.split * tiles;
+    item.splits = splits;
+    item.c0 = item.split * w.k_chunks / splits;
+    item.nc = (item.split + 1) * w.k_chunks / splits - item.c0;
+    return true;
+}
+template <int BM, int BN>
+__global__ __launch_bounds__(256, 2) void wgrad_batch_kernel(WgradBatch w) {
+    using TA = TileKS64<BM>;
+    using TB = TileKS64<BN>;
+    constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32;
+    constexpr int LA = TA::LOADS, LB = TB::LOADS, LOADS = LA + LB;
+    constexpr int SLOT = TA::BYTES + TB::BYTES;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t smem_base = lds_address(smem);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+
+    // ---- producer: one stage ahead of the consumer, across the block's (at most two) items --------------
+    int p_group = 0, p_left = 0, p_slot = 0;
+    const bf16_t *pa[LA], *pb[LB];
+    int64_t a_step = 0, b_step = 0;
+    auto producer_open = [&]() { // the next group that has an item for this block; false when there is none
+        WgradItem item;
+        while (p_group < 2 && !wgrad_item(w, p_group, blockIdx.x, item))
+            ++p_group;
+        if (p_group >= 2)
+            return false;
+        ++p_group;
+        p_left = item.nc;
+        const WgradTile t = wgrad_tile<BM, BN>(w, item.tile);
+        const int lda = w.lddy[t.job], ldb = w.ldx[t.job];
+        a_step = TA::step(lda), b_step = TB::step(ldb);
+        const bf16_t *a0 = w.dy[t.job] + TA::origin(t.m0, item.c0 * 64, lda);
+        const bf16_t *b0 = w.x[t.job] + TB::origin(t.n0, item.c0 * 64, ldb);
+#pragma unroll
+        for (int j = 0; j < LA; ++j)
+            pa[j] = a0 + TA::source_offset(j, tid, lda);
+#pragma unroll
+        for (int j = 0; j < LB; ++j)
+            pb[j] = b0 + TB::source_offset(j, tid, ldb);
+        return true;
+    };
+    auto copy_one = [&](int n) {
+        const uint32_t to = smem_base + uint32_t(p_slot) * SLOT;
+        if (n < LA) {
+            async_copy16(__builtin_amdgcn_readfirstlane(to + TA::lds_offset(n, tid)), pa[n]);
+            pa[n] += a_step;
+        } else {
+            async_copy16(__builtin_amdgcn_readfirstlane(to + TA::BYTES + TB::lds_offset(n - LA, tid)), pb[n - LA]);
+            pb[n - LA] += b_step;
+        }
+    };
+    if (!producer_open())
+        return;
+#pragma unroll
+    for (int n = 0; n < LOADS; ++n)
+        copy_one(n);
+    --p_left;
+    p_slot = 1;
+
+    int c_slot = 0;
+    for (int group = 0; group < 2; ++group) {
+        WgradItem item;
+        if (!wgrad_item(w, group, blockIdx.x, item))
+            continue;
+        f32x16 acc[FM][FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[i][j][r] = 0.f;
+        for (int c = 0; c < item.nc; ++c) {
+            wait_vmcnt<0>();
+            __syncthreads();
+            bool copy = true;
+            if (p_left == 0)
+                copy = producer_open();
+            multiply_stage<TA, TB, FM, FN, LOADS>(acc, smem + c_slot * SLOT, wm, wn, lane, copy, copy_one);
+            if (copy) {
+                --p_left;
+                p_slot ^= 1;
+            }
+            c_slot ^= 1;
+        }
+        __syncthreads(); // the transposition buffers lie in the stage consumed last
+        unsigned char *mine = smem + (c_slot ^ 1) * SLOT + wave * 4096;
+        if (item.splits == 1) {
+            const WgradTile t = wgrad_tile<BM, BN>(w, item.tile);
+            const EpilogueF32 whole{w.dw[t.job], w.lddw[t.job], 0, w.accumulate};
+            staged_store_f32<FM, FN>(acc, mine, whole, t.m0 + wm, t.n0 + wn, lane, 0);
+        } else {
+            const EpilogueF32 piece{w.pieces + size_t(piece_slot(w, item.tile, item.split)) * (BM * BN), BN, 0, 0};
+            staged_store_f32<FM, FN>(acc, mine, piece, wm, wn, lane, 0);
+        }
+    }
+    wait_vmcnt<0>();
+}
+// Sums the pieces of every split tile, in split order, into the gradient.  Four blocks per tile, 32 rows each.
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void wgrad_batch_fold_kernel(WgradBatch w) {
+    const int tile = blockIdx.x >> 2, part = blockIdx.x & 3;
+    const int splits = tile < w.tiles_a ? w.splits_a : w.splits_b;
+    if (splits == 1)
+        return; // the tile's only item wrote the gradient itself
+    const WgradTile t = wgrad_tile<BM, BN>(w, tile);
+    float *out = w.dw[t.job];
+    const int ld = w.lddw[t.job];
+    const float *first = w.pieces + size_t(piece_slot(w, tile, 0)) * (BM * BN);
+    constexpr int QUADS = BN / 4, ROWS = BM / 4;
+    for (int i = threadIdx.x; i < ROWS * QUADS; i += 256) {
+        const int r = part * ROWS + i / QUADS, c = (i % QUADS) * 4;
+        float4 sum = make_float4(0, 0, 0, 0);
+        for (int split = 0; split < splits; ++split) { // fixed order
+            const float4 v = *reinterpret_cast<const float4 *>(first + size_t(split) * (BM * BN) + r * BN + c);
+            sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+        }
+        float4 *p = reinterpret_cast<float4 *>(out + size_t(t.m0 + r) * ld + t.n0 + c);
+        if (w.accumulate) {
+            const float4 old = *p;
+            sum.x += old.x, sum.y += old.y, sum.z += old.z, sum.w += old.w;
+        }
+        *p = sum;
+    }
 }
 
 // Sums split-K slabs in a fixed order (deterministic) into the fp32 gradient.
@@ -913,5 +1101,105 @@ extern "C" int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uin
                            static_cast<const float *>(workspace), size_t(N) * K, splits, dW, N, K, lddw,
                            accumulate);
         check_hip(hipGetLastError(), "split-K reduce launch: ");
+    });
+}
+
+namespace {
+// Job table and the two tile groups of a batch.
+bool plan_wgrad_batch(int M, int count, const TgkWgradJob *jobs, WgradBatch &w, std::string &why) {
+    if (count < 1 || count > MAX_WGRAD_JOBS || !jobs) {
+        why = "gemm_wgrad_batch: between 1 and 4 jobs";
+        return false;
+    }
+    if (M <= 0 || M % 64) {
+        why = "gemm_wgrad_batch: M (the reduced dimension) must be a multiple of 64";
+        return false;
+    }
+    w = WgradBatch{};
+    w.count = count;
+    w.k_chunks = M / 64;
+    for (int j = 0; j < count; ++j) {
+        const TgkWgradJob &job = jobs[j];
+        if (job.N <= 0 || job.K <= 0 || job.N % 128 || job.K % 192) {
+            why = "gemm_wgrad_batch: every N must be a multiple of 128 and every K of 192";
+            return false;
+        }
+        w.dy[j] = job.dY, w.x[j] = job.X, w.dw[j] = job.dW;
+        w.lddy[j] = job.lddy, w.ldx[j] = job.ldx, w.lddw[j] = job.lddw;
+        w.tiles_n[j] = job.K / 192;
+        w.first_tile[j + 1] = w.first_tile[j] + (job.N / 128) * (job.K / 192);
+    }
+    // Two groups of tiles, each split so that it makes (up to) one item per resident block: the first
+    // blocks / ceil(blocks / tiles) tiles ceil(blocks / tiles) ways, the rest as many ways as fill the blocks
+    // again (items of at least four chunks).
+    const int tiles = w.first_tile[count], blocks = resident_blocks(TILE_128x192);
+    const int max_splits = w.k_chunks / 4 > 0 ? w.k_chunks / 4 : 1;
+    int splits_a = (blocks + tiles - 1) / tiles;
+    if (splits_a > max_splits)
+        splits_a = max_splits;
+    int tiles_a = blocks / splits_a;
+    if (tiles_a > tiles)
+        tiles_a = tiles;
+    const int tiles_b = tiles - tiles_a;
+    int splits_b = tiles_b ? blocks / tiles_b : 1;
+    if (splits_b > max_splits)
+        splits_b = max_splits;
+    if (splits_b < 1)
+        splits_b = 1;
+    w.tiles_a = tiles_a, w.splits_a = splits_a, w.tiles_b = tiles_b, w.splits_b = splits_b;
+    return true;
+}
+int wgrad_batch_blocks(const WgradBatch &w) {
+    const int a = w.tiles_a * w.splits_a, b = w.tiles_b * w.splits_b;
+    return a > b ? a : b;
+}
+size_t wgrad_batch_pieces(const WgradBatch &w) {
+    return size_t(w.tiles_a * w.splits_a + w.tiles_b * w.splits_b) * 128 * 192 * sizeof(float);
+}
+} // namespace
+
+extern "C" size_t tgk_gemm_wgrad_batch_workspace(int M, int count, const TgkWgradJob *jobs) {
+    try {
+        WgradBatch w;
+        std::string why;
+        return plan_wgrad_batch(M, count, jobs, w, why) ? wgrad_batch_pieces(w) : 0;
+    } catch (...) {
+        return 0;
+    }
+}
+
+extern "C" int tgk_gemm_wgrad_batch(hipStream_t stream, int M, int count, const TgkWgradJob *jobs, int accumulate,
+                                    void *workspace, size_t workspace_bytes) {
+    return guarded([&] {
+        WgradBatch w;
+        std::string why;
+        if (!plan_wgrad_batch(M, count, jobs, w, why))
+            throw std::invalid_argument(why);
+        for (int j = 0; j < count; ++j) {
+            check_operand(jobs[j].dY, jobs[j].lddy, "dY");
+            check_operand(jobs[j].X, jobs[j].ldx, "X");
+            require(jobs[j].lddy >= jobs[j].N && jobs[j].ldx >= jobs[j].K, "gemm_wgrad_batch: leading dimension too small");
+            require(jobs[j].dW && !(reinterpret_cast<uintptr_t>(jobs[j].dW) & 15) && jobs[j].lddw % 4 == 0 &&
+                        jobs[j].lddw >= jobs[j].K,
+                    "gemm_wgrad_batch: dW must be 16-byte aligned with leading dimension % 4 == 0");
+        }
+        require(workspace && workspace_bytes >= wgrad_batch_pieces(w) && !(reinterpret_cast<uintptr_t>(workspace) & 15),
+                "gemm_wgrad_batch: workspace too small (see tgk_gemm_wgrad_batch_workspace)");
+        w.accumulate = accumulate;
+        w.pieces = static_cast<float *>(workspace);
+        auto kernel = wgrad_batch_kernel<128, 192>;
+        constexpr size_t lds = 2 * (128 + 192) * 128;
+        static std::atomic<bool> configured[MAX_DEVICES];
+        const int device = current_device();
+        if (!configured[device].load(std::memory_order_acquire)) {
+            check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)),
+                      "gemm LDS size: ");
+            configured[device].store(true, std::memory_order_release);
+        }
+        hipLaunchKernelGGL(kernel, dim3(wgrad_batch_blocks(w)), dim3(256), lds, stream, w);
+        check_hip(hipGetLastError(), "wgrad batch launch: ");
+        hipLaunchKernelGGL((wgrad_batch_fold_kernel<128, 192>), dim3(w.first_tile[count] * 4), dim3(256), 0, stream, w);
+        check_hip(hipGetLastError(), "wgrad batch fold launch: ");
     });
 }
