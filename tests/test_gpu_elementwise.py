@@ -85,6 +85,14 @@ def test_layernorm_forward_backward(orc, M, D):
         base = 2.0 if residual else 0.0  # accumulate flag follows residual in this test
         assert rel(host(dg) - base, want_dg) < 1e-4
         assert rel(host(db) - base, want_db) < 1e-4
+        # the same with the residual gradient read from a buffer of its own, which stays untouched
+        apart = torch.empty_like(dx)
+        check(lib.tgk_layernorm_bwd_add(stream(), M, D, x.data_ptr(), dy.data_ptr(), gh.data_ptr(), gl.data_ptr(),
+                                        prior.data_ptr() if residual else None, apart.data_ptr(), dg.data_ptr(),
+                                        db.data_ptr(), 1e-5, 0, ws.data_ptr(), need))
+        sync()
+        assert torch.equal(apart, dx)
+        assert np.array_equal(host(prior), ph)
 
 
 def test_cross_entropy_loss_logits_and_gradient(orc):
