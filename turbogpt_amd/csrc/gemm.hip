@@ -1,25 +1,28 @@
 // bf16 MFMA GEMM family for gfx950: forward Y = X W^T, dgrad dX = dY W, wgrad dW = dY^T X.
 // Replaces project / matmul+cast_result / weight_gradient of the reference
 // (cuda/mma.cuh:77-108, cuda/ops.cuh:30-55, cuda/ops.cuh:83-109) and, through the fixed-order
-// split-K fold, reduce_gradients (cuda/trainer.cuh:9-47).
+// folds of split-K pieces, reduce_gradients (cuda/trainer.cuh:9-47).
 //
-// One kernel template computes C[m][n] = sum_k A(m,k) B(n,k).  Each operand is either
-// "k-contiguous" (stored [row][k]) or "k-strided" (stored [k][row]):
-//   forward : A = X  [M][K] k-contiguous, B = W  [N][K] k-contiguous
-//   dgrad   : A = dY [M][N] k-contiguous, B = W  [N][K] read as (n = K index, k = N index): k-strided
+// Every kernel computes C[m][n] = sum_k A(m,k) B(n,k).  Each operand is either "k-contiguous" (stored
+// [row][k]) or "k-strided" (stored [k][row]):
+//   forward : A = X  [M][K] k-contiguous, B = W [N][K] k-contiguous
+//   dgrad   : A = dY [M][N] k-contiguous, B = the transposed weight Wt [K][N] k-contiguous (tgk_gemm_dgrad_t),
+//             or W [N][K] read as (n = K index, k = N index): k-strided (tgk_gemm_dgrad)
 //   wgrad   : A = dY [M][N] k-strided (m = out index), B = X [M][K] k-strided, fp32 out, split-K
 //
 // Data path: global -> LDS directly (global_load_lds_dwordx4: no staging registers, no LDS store
-// instructions), S stages of 32 k deep; the copies run S-1 k-tiles ahead of the MFMAs and keep
-// running across tile boundaries, because a block is persistent and walks a list of work items
-// (tile x split).  LDS tiles are unpadded and XOR-swizzled on 16-byte chunks (a wave-wide copy fills
-// 1 KiB of LDS contiguously, so padding is not available); measured bank conflicts are zero.
-// k-contiguous tiles give each MFMA fragment with one ds_read_b128; k-strided tiles keep the
-// natural [k][row] image and are read with the transposing ds_read_b64_tr_b16.
-// 256 threads = 2x2 waves of v_mfma_f32_32x32x16_bf16; the instruction's A operand is fed with
-// *our B rows* so that a lane ends up holding 4 consecutive n for one m: 8-byte bf16 / 16-byte
-// fp32 stores and a fused epilogue on the fragment.  Fragments of the next k-step are read while
-// the current MFMAs run, also across the per-k-tile barrier.
+// instructions); the copies keep running across tile boundaries, because a block is persistent and walks a
+// list of work items (tile x split).  LDS tiles are unpadded and XOR-swizzled on 16-byte chunks (a wave-wide
+// copy fills 1 KiB of LDS contiguously, so padding is not available); measured bank conflicts are zero.
+// k-contiguous tiles give each MFMA fragment with one ds_read_b128; k-strided tiles keep the natural [k][row]
+// image and are read with the transposing ds_read_b64_tr_b16.  256 threads = 2x2 waves of
+// v_mfma_f32_32x32x16_bf16; the instruction's A operand is fed with *our B rows* so that a lane ends up holding
+// 4 consecutive n for one m.  Results leave through a wave-private LDS transposition so that stores cover
+// whole row pieces, with the residual / GELU / GELU' epilogues applied in that layout.
+//
+// Three kernels: gemm64_kernel (two stages of 64 k, copies placed between the MFMAs: every training shape),
+// gemm_kernel (S stages of 32 k: the shapes gemm64_kernel does not take), wgrad_batch_kernel (the weight
+// gradients of several matrices in one launch).
 #include "common.h"
 #include <atomic>
 #include "../../include/tgk_kernels.h"
