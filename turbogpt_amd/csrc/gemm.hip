@@ -920,13 +920,13 @@ void dispatch_gemm(hipStream_t stream, Tile tile, const bf16_t *A, int lda, cons
         launch_gemm<128, 128, 4, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, blocks, epilogue);
 }
 
-// 128x192 tiles with the reduced dimension a multiple of 64 take the two-stage 64-k kernel.
-bool takes_64(Tile tile, int reduced) { return tile == TILE_128x192 && reduced % 64 == 0; }
+// A reduced dimension that is a multiple of 64 takes the two-stage 64-k kernel.
+bool takes_64(Tile tile, int reduced) { return tile != TILE_NONE && reduced % 64 == 0; }
 
-template <bool AKC, bool BKC, class Epilogue>
-void launch_gemm64(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
-                   int splits, const Epilogue &epilogue) {
-    constexpr int BM = 128, BN = 192;
+template <int BN, bool AKC, bool BKC, class Epilogue>
+void launch_gemm64_tile(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
+                        int splits, const Epilogue &epilogue) {
+    constexpr int BM = 128;
     auto kernel = gemm64_kernel<BM, BN, AKC, BKC, Epilogue>;
     constexpr size_t lds = 2 * (BM + BN) * 128;
     static std::atomic<bool> configured[MAX_DEVICES];
@@ -943,6 +943,14 @@ void launch_gemm64(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, A, lda, B, ldb, K / 64, splits, tiles_n, tiles,
                        splits == 1 ? xcd_columns(tiles_m, tiles_n, BM, BN, K, blocks) : 1, epilogue);
     check_hip(hipGetLastError(), "gemm launch: ");
+}
+template <bool AKC, bool BKC, class Epilogue>
+void launch_gemm64(hipStream_t stream, Tile tile, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N,
+                   int K, int splits, const Epilogue &epilogue) {
+    if (tile == TILE_128x192)
+        launch_gemm64_tile<192, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
+    else
+        launch_gemm64_tile<128, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
 }
 
 void check_operand(const void *p, int ld, const char *name) {
@@ -983,7 +991,7 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
             e.out2 = gelu_out, e.ld_out2 = ldg, e.mode = EPI_GELU;
         }
         if (takes_64(tile, K))
-            launch_gemm64<true, true>(stream, X, ldx, W, ldw, M, N, K, 1, e);
+            launch_gemm64<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, 1, e);
         else
             dispatch_gemm<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, 1, e);
     });
@@ -1053,7 +1061,7 @@ extern "C" int tgk_gemm_dgrad_t(hipStream_t stream, int M, int N, int K, const u
         }
         // C[m][i] = sum_o dY[m][o] Wt[i][o]: the forward product with (rows, reduced) = (K, N)
         if (takes_64(tile, N))
-            launch_gemm64<true, true>(stream, dY, lddy, Wt, ldwt, M, K, N, 1, e);
+            launch_gemm64<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, 1, e);
         else
             dispatch_gemm<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, 1, e);
     });
@@ -1084,8 +1092,8 @@ extern "C" int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uin
         const int splits = wgrad_splits(tile, (N / tile_rows(tile)) * (K / tile_cols(tile)), M / BK);
         if (splits == 1) {
             EpilogueF32 e{dW, lddw, 0, accumulate};
-            if (takes_64(tile, M))
-                launch_gemm64<false, false>(stream, dY, lddy, X, ldx, N, K, M, 1, e);
+            if (tile == TILE_128x192 && takes_64(tile, M)) // 128x128 weight-gradient tiles measured faster in 32-k stages
+                launch_gemm64<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, 1, e);
             else
                 dispatch_gemm<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, 1, e);
             return;
@@ -1094,8 +1102,8 @@ extern "C" int tgk_gemm_wgrad(hipStream_t stream, int M, int N, int K, const uin
         require(workspace && workspace_bytes >= need && !(reinterpret_cast<uintptr_t>(workspace) & 15),
                 "gemm_wgrad: workspace too small (see tgk_gemm_wgrad_workspace)");
         EpilogueF32 e{static_cast<float *>(workspace), K, size_t(N) * K, 0};
-        if (takes_64(tile, M))
-            launch_gemm64<false, false>(stream, dY, lddy, X, ldx, N, K, M, splits, e);
+        if (tile == TILE_128x192 && takes_64(tile, M))
+            launch_gemm64<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, splits, e);
         else
             dispatch_gemm<false, false>(stream, tile, dY, lddy, X, ldx, N, K, M, splits, e);
         const size_t quads = size_t(N) * K / 4;
