@@ -152,6 +152,24 @@ def kernel_sweeps(out):
             print(json.dumps({"kernel": f"gemm_{name}", "M": M, "K": k, "N": n, "ms": round(ms, 4),
                               "tflops": round(flop / ms / 1e9, 1),
                               "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
+    # the four weight gradients of one block in one launch, as the engine runs them
+    import ctypes
+    from turbogpt_amd.bridge import WgradJob
+    shapes = [(D, F), (F, D), (D, D), (3 * D, D)]
+    keep, jobs = [], (WgradJob * 4)()
+    for j, (n, k) in enumerate(shapes):
+        dy = torch.randn(M, n, device="cuda").bfloat16()
+        x = torch.randn(M, k, device="cuda").bfloat16()
+        dw = torch.empty(n, k, device="cuda")
+        keep.append((dy, x, dw))
+        jobs[j] = WgradJob(n, k, dy.data_ptr(), n, x.data_ptr(), k, dw.data_ptr(), k)
+    need = lib.tgk_gemm_wgrad_batch_workspace(M, 4, ctypes.addressof(jobs))
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ms = timed(lambda: check(lib.tgk_gemm_wgrad_batch(stream, M, 4, ctypes.addressof(jobs), 0, ws.data_ptr(), need)))
+    flop = sum(2.0 * M * n * k for n, k in shapes)
+    print(json.dumps({"kernel": "gemm_wgrad_batch", "M": M, "shapes_N_K": shapes, "ms": round(ms, 4),
+                      "tflops": round(flop / ms / 1e9, 1),
+                      "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
     d = H * 64
     qkv = torch.randn(M, 3 * d, device="cuda").bfloat16()
     do = torch.randn(M, d, device="cuda").bfloat16()
