@@ -344,22 +344,29 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
                 s = mfma(qrows.load(qt_tile, qt, ks), kf[ks], s);
                 dp = mfma(qrows.load(gt_tile, qt, ks), vf[ks], dp);
             }
-            const bool diagonal = qh < wave_k0 + 31;
+            // the causal mask costs three instructions per score: only in the half tiles that straddle the
+            // diagonal (a wave-uniform branch; as a per-element condition it is paid everywhere)
+            auto probabilities = [&](auto masked) {
 #pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const int at = qt * 32 + 8 * q4 + 4 * g;
-                const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][0][at]);
-                const f32x4 del4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][1][at]);
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const int at = qt * 32 + 8 * q4 + 4 * g;
+                    const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][0][at]);
+                    const f32x4 del4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][1][at]);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = q4 * 4 + e;
-                    float p = exp2_fast(fmaf(s[r], c, -lse4[e]));
-                    if (diagonal && krow > q0 + at + e)
-                        p = 0.f;
-                    s[r] = p;
-                    dp[r] = p * (dp[r] - del4[e]);
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = q4 * 4 + e;
+                        float p = exp2_fast(fmaf(s[r], c, -lse4[e]));
+                        if (decltype(masked)::value && krow > q0 + at + e)
+                            p = 0.f;
+                        s[r] = p;
+                        dp[r] = p * (dp[r] - del4[e]);
+                    }
                 }
-            }
+            };
+            if (qh < wave_k0 + 31)
+                probabilities(Const<1>{});
+            else
+                probabilities(Const<0>{});
 #pragma unroll
             for (int kk2 = 0; kk2 < 2; ++kk2) {
                 const bf16x8 pf = acc_to_frag(s, kk2);
@@ -484,13 +491,20 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
                 s = mfma(krows.load(kt, mt, ks), qf[ks], s);
                 dp = mfma(krows.load(vt, mt, ks), gf[ks], dp);
             }
+            // the causal mask only in the tiles that straddle the diagonal (wave-uniform branch)
+            auto probabilities = [&](auto masked) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float p = exp2_fast(fmaf(s[r], c, -lse));
-                if (diagonal && kv0 + mt * 32 + acc_row(r, g) > qrow)
-                    p = 0.f;
-                dp[r] = p * (dp[r] - del);
-            }
+                for (int r = 0; r < 16; ++r) {
+                    float p = exp2_fast(fmaf(s[r], c, -lse));
+                    if (decltype(masked)::value && kv0 + mt * 32 + acc_row(r, g) > qrow)
+                        p = 0.f;
+                    dp[r] = p * (dp[r] - del);
+                }
+            };
+            if (diagonal)
+                probabilities(Const<1>{});
+            else
+                probabilities(Const<0>{});
 #pragma unroll
             for (int kk2 = 0; kk2 < 2; ++kk2) {
                 const bf16x8 dsf = acc_to_frag(dp, kk2);
