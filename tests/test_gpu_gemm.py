@@ -169,7 +169,8 @@ def run_wgrad_batch(M, shapes, rng, accumulate=0, start=0.0):
 
 @pytest.mark.parametrize("M,shapes", [(64, [(128, 192)]), (256, [(128, 192), (256, 384)]),
                                       (2048, [(768, 768), (256, 192), (128, 576), (384, 192)]),
-                                      (4096, [(128, 192), (128, 192), (128, 192)])])
+                                      (4096, [(128, 192), (128, 192), (128, 192)]),
+                                      (128, [(2560, 1920), (2560, 1920), (2560, 1920)])])  # more tiles than blocks
 def test_wgrad_batch_against_the_checker(orc, M, shapes):
     """Several weight gradients in one launch: every job against the checker, accumulate, and a second run
     bit-identical (runs and pieces are summed in a fixed order)."""
