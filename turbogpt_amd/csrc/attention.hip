@@ -63,12 +63,19 @@ TG_DEVICE int swz(int row) {
     return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
 }
 // this wave's two copies (regions wave and wave+4, 8 rows each) of a 64-row tile starting at `base`
+TG_DEVICE void tile_copy_async_one(uint32_t lds_tile, const bf16_t *base, int ld, int wave, int lane, int j) {
+    const int region = wave + 4 * j, row = region * 8 + (lane >> 3), chunk = (lane & 7) ^ swz(row);
+    async_copy16(__builtin_amdgcn_readfirstlane(lds_tile + region * 1024), base + size_t(row) * ld + chunk * 8);
+}
+// byte offset of this lane's 16 bytes within a 64-row tile whose rows are ld elements apart
+TG_DEVICE uint32_t tile_copy_offset(int ld, int wave, int lane, int j) {
+    const int region = wave + 4 * j, row = region * 8 + (lane >> 3), chunk = (lane & 7) ^ swz(row);
+    return uint32_t(row * ld + chunk * 8) * 2;
+}
 TG_DEVICE void tile_copy_async(uint32_t lds_tile, const bf16_t *base, int ld, int wave, int lane) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int region = wave + 4 * j, row = region * 8 + (lane >> 3), chunk = (lane & 7) ^ swz(row);
-        async_copy16(__builtin_amdgcn_readfirstlane(lds_tile + region * 1024), base + size_t(row) * ld + chunk * 8);
-    }
+    for (int j = 0; j < 2; ++j)
+        tile_copy_async_one(lds_tile, base, ld, wave, lane, j);
 }
 // The swizzle terms of both fragment kinds depend on the lane only (swz(row + 32) = swz(row);
 // swz(r + 16) = swz(r)), so a kernel computes these element offsets once and adds compile-time
@@ -139,6 +146,25 @@ TG_DEVICE float halves_sum(float x) {
     const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
     return __uint_as_float(both[0]) + __uint_as_float(both[1]);
 }
+// Writes a 32 x 32 accumulator whose rows (lane % 32) are rows of memory: `row` points at this lane's row, first
+// of the 32 columns.  Lane l holds columns 8*q4 + 4*g + {0..3} (registers 4*q4 ..) of its row, lane l + 32 the
+// other four of every eight.  The two trade halves, so that one ends up with columns 0..15 and the other with
+// 16..31 and each writes 32 contiguous bytes: a quarter of the store instructions and of the cache lines touched
+// per instruction that 8-byte pieces take.
+TG_DEVICE void store_acc_rows(bf16_t *row, const f32x16 &acc, float scale, int g) {
+    uint32_t x[4], y[4];
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) {
+        x[q4] = pack_bf16(acc[q4 * 4 + 0] * scale, acc[q4 * 4 + 1] * scale);
+        y[q4] = pack_bf16(acc[q4 * 4 + 2] * scale, acc[q4 * 4 + 3] * scale);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const auto ax = __builtin_amdgcn_permlane32_swap(x[h], x[h + 2], false, false);
+        const auto ay = __builtin_amdgcn_permlane32_swap(y[h], y[h + 2], false, false);
+        *reinterpret_cast<u32x4 *>(row + 16 * g + 8 * h) = u32x4{ax[0], ay[0], ax[1], ay[1]};
+    }
+}
 
 // ---------------------------------------------------------------------------------------------
 // forward: block = 128 queries (4 waves x 32), key/value tiles of 64 in three LDS stages filled by
@@ -193,10 +219,13 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restri
         else
             wait_vmcnt<0>();
         __syncthreads(); // tile j visible to every wave; everyone is done with tile j-1's stage
-        if (j + 2 < tiles)
-            produce((STAGE + 2) % 3, j + 2);
-        if (j >= my_tiles)
+        // the copies of tile j+2 go out at the end of the step, where the waves have drifted apart: behind
+        // the barrier every wave of the CU would queue its copies at the same moment
+        if (j >= my_tiles) {
+            if (j + 2 < tiles)
+                produce((STAGE + 2) % 3, j + 2);
             return;
+        }
         const bf16_t *kt = stages[STAGE][0], *vt = stages[STAGE][1];
         const int kv0 = j * 64;
         f32x16 s[2] = {zero16(), zero16()};
@@ -247,6 +276,8 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restri
             for (int dt = 0; dt < 2; ++dt)
                 o[dt] = mfma(vcols.load(vt, kk, dt), pf, o[dt]);
         }
+        if (j + 2 < tiles)
+            produce((STAGE + 2) % 3, j + 2);
     };
     for (int j = 0; j < tiles; j += 3) { // tiles is block uniform
         step(Const<0>{}, j);
@@ -257,16 +288,10 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restri
     }
     l = halves_sum(l);
     const float inv = 1.0f / l;
-    bf16_t *op = O + (token0 + qrow) * ldo + h * HD + 4 * g;
+    bf16_t *op = O + (token0 + qrow) * ldo + h * HD;
 #pragma unroll
     for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            u32x2 packed;
-            packed.x = pack_bf16(o[dt][q4 * 4 + 0] * inv, o[dt][q4 * 4 + 1] * inv);
-            packed.y = pack_bf16(o[dt][q4 * 4 + 2] * inv, o[dt][q4 * 4 + 3] * inv);
-            *reinterpret_cast<u32x2 *>(op + dt * 32 + q4 * 8) = packed;
-        }
+        store_acc_rows(op + dt * 32, o[dt], inv, g);
     if (g == 0)
         LSE[(size_t(b) * H + h) * T + qrow] = (m + __log2f(l)) * LN2;
 }
@@ -298,15 +323,26 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
     const bf16_t *gbase = dO + (token0 + first * 64) * lddo + h * HD;
     const float *row_source = ((wave & 1) ? delta : lse2) + (size_t(b) * H + h) * T + first * 64 + lane;
     const uint32_t lds0 = lds_address(&stages[0][0][0]), rows0 = lds_address(&rows[0][wave & 1][0]);
-    auto produce = [&](int stage, int j) { // five copies per wave
+    const uint32_t q_offset[2] = {tile_copy_offset(ld, wave, lane, 0), tile_copy_offset(ld, wave, lane, 1)};
+    const uint32_t g_offset[2] = {tile_copy_offset(lddo, wave, lane, 0), tile_copy_offset(lddo, wave, lane, 1)};
+    auto produce_one = [&](int stage, int j, int n) { // n-th of a wave's five copies for tile j
         const uint32_t slot = lds0 + uint32_t(stage) * (2 * TILE_ELEMS * 2);
-        tile_copy_async(slot, qbase + size_t(j) * 64 * ld, ld, wave, lane);
-        tile_copy_async(slot + TILE_ELEMS * 2, gbase + size_t(j) * 64 * lddo, lddo, wave, lane);
-        async_copy4(__builtin_amdgcn_readfirstlane(rows0 + uint32_t(stage) * (2 * 64 * 4)), row_source + j * 64);
+        if (n < 2)
+            async_copy16(__builtin_amdgcn_readfirstlane(slot + (wave + 4 * n) * 1024), qbase + size_t(j) * 64 * ld,
+                         q_offset[n]);
+        else if (n < 4)
+            async_copy16(__builtin_amdgcn_readfirstlane(slot + TILE_ELEMS * 2 + (wave + 4 * (n - 2)) * 1024),
+                         gbase + size_t(j) * 64 * lddo, g_offset[n - 2]);
+        else
+            async_copy4(__builtin_amdgcn_readfirstlane(rows0 + uint32_t(stage) * (2 * 64 * 4)), row_source + j * 64);
+    };
+    auto produce = [&](int stage, int j) {
+#pragma unroll
+        for (int n = 0; n < 5; ++n)
+            produce_one(stage, j, n);
     };
     produce(0, 0);
-    if (tiles > 1)
-        produce(1, 1);
+    produce(1, tiles > 1 ? 1 : 0);
 
     bf16x8 kf[4], vf[4];
     {
@@ -324,20 +360,20 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
 
     auto step = [&](auto stage_tag, int j) {
         constexpr int STAGE = decltype(stage_tag)::value;
-        if (j + 1 < tiles)
-            wait_vmcnt<5>(); // only tile j+1's copies may still be in flight
-        else
-            wait_vmcnt<0>();
+        wait_vmcnt<5>(); // only the five copies issued during tile j-1 may still be in flight
         __syncthreads(); // tile j visible to every wave; everyone is done with tile j-1's stage
-        if (j + 2 < tiles)
-            produce((STAGE + 2) % 3, j + 2);
+        // The copies of tile j+2 go out at the end of the step, where the waves have drifted apart: behind the
+        // barrier all eight waves of the CU queue theirs at once and wait for one another (measured -2 %).
+        // Every step issues five (past the end the last tile once more, into the stage nobody reads any
+        // more), so the wait above is always the same.
+        const int ahead = j + 2 < tiles ? j + 2 : tiles - 1;
         const bf16_t *qt_tile = stages[STAGE][0], *gt_tile = stages[STAGE][1];
         const int q0 = (first + j) * 64;
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+        auto half = [&](auto half_tag) {
+            constexpr int qt = decltype(half_tag)::value;
             const int qh = q0 + qt * 32;
             if (qh + 31 < wave_k0) // every query of this half precedes this wave's keys (wave uniform)
-                continue;
+                return;
             f32x16 s = zero16(), dp = zero16();
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
@@ -377,7 +413,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
                     dk[dt] = mfma(qcols.load(qt_tile, qt * 2 + kk2, dt), dsf, dk[dt]);
                 }
             }
-        }
+        };
+        half(Const<0>{});
+        half(Const<1>{});
+        produce((STAGE + 2) % 3, ahead);
     };
     for (int j = 0; j < tiles; j += 3) { // tiles is block uniform
         step(Const<0>{}, j);
@@ -386,20 +425,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
         if (j + 2 < tiles)
             step(Const<2>{}, j + 2);
     }
-    bf16_t *kp = dK + (token0 + krow) * lddq + h * HD + 4 * g;
-    bf16_t *vp = dV + (token0 + krow) * lddq + h * HD + 4 * g;
+    wait_vmcnt<0>(); // no copy may land in LDS after the block has left
+    bf16_t *kp = dK + (token0 + krow) * lddq + h * HD;
+    bf16_t *vp = dV + (token0 + krow) * lddq + h * HD;
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            u32x2 pk, pv;
-            pk.x = pack_bf16(dk[dt][q4 * 4 + 0] * scale, dk[dt][q4 * 4 + 1] * scale);
-            pk.y = pack_bf16(dk[dt][q4 * 4 + 2] * scale, dk[dt][q4 * 4 + 3] * scale);
-            pv.x = pack_bf16(dv[dt][q4 * 4 + 0], dv[dt][q4 * 4 + 1]);
-            pv.y = pack_bf16(dv[dt][q4 * 4 + 2], dv[dt][q4 * 4 + 3]);
-            *reinterpret_cast<u32x2 *>(kp + dt * 32 + q4 * 8) = pk;
-            *reinterpret_cast<u32x2 *>(vp + dt * 32 + q4 * 8) = pv;
-        }
+    for (int dt = 0; dt < 2; ++dt) {
+        store_acc_rows(kp + dt * 32, dk[dt], scale, g);
+        store_acc_rows(vp + dt * 32, dv[dt], 1.0f, g);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -474,10 +507,13 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
         else
             wait_vmcnt<0>();
         __syncthreads();
-        if (j + 2 < tiles)
-            produce((STAGE + 2) % 3, j + 2);
-        if (j >= my_tiles)
+        // the copies of tile j+2 go out at the end of the step, where the waves have drifted apart: behind
+        // the barrier every wave of the CU would queue its copies at the same moment
+        if (j >= my_tiles) {
+            if (j + 2 < tiles)
+                produce((STAGE + 2) % 3, j + 2);
             return;
+        }
         const bf16_t *kt = stages[STAGE][0], *vt = stages[STAGE][1];
         const int kv0 = j * 64;
         const bool diagonal = kv0 + 63 > wave_q0;
@@ -513,6 +549,8 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
                     dq[dt] = mfma(kcols.load(kt, mt * 2 + kk2, dt), dsf, dq[dt]);
             }
         }
+        if (j + 2 < tiles)
+            produce((STAGE + 2) % 3, j + 2);
     };
     for (int j = 0; j < tiles; j += 3) { // tiles is block uniform
         step(Const<0>{}, j);
@@ -521,16 +559,10 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
         if (j + 2 < tiles)
             step(Const<2>{}, j + 2);
     }
-    bf16_t *qp = dQ + (token0 + qrow) * lddq + h * HD + 4 * g;
+    bf16_t *qp = dQ + (token0 + qrow) * lddq + h * HD;
 #pragma unroll
     for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            u32x2 packed;
-            packed.x = pack_bf16(dq[dt][q4 * 4 + 0] * scale, dq[dt][q4 * 4 + 1] * scale);
-            packed.y = pack_bf16(dq[dt][q4 * 4 + 2] * scale, dq[dt][q4 * 4 + 3] * scale);
-            *reinterpret_cast<u32x2 *>(qp + dt * 32 + q4 * 8) = packed;
-        }
+        store_acc_rows(qp + dt * 32, dq[dt], scale, g);
 }
 
 void check_attention_shape(int B, int H, int T, int hd) {

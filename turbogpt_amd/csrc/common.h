@@ -90,6 +90,11 @@ TG_DEVICE float wave_max(float x) {
 TG_DEVICE void async_copy16(uint32_t lds_base, const void *global) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(global) : "memory");
 }
+// the same copy from a wave-uniform base plus a 32-bit byte offset per lane: one address register instead of two
+TG_DEVICE void async_copy16(uint32_t lds_base, const void *uniform_base, uint32_t lane_offset) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_offset), "s"(uniform_base)
+                 : "memory");
+}
 // the 4-byte form: lane l lands at lds_base + 4*l
 TG_DEVICE void async_copy4(uint32_t lds_base, const void *global) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(global) : "memory");
