@@ -785,20 +785,39 @@ __global__ __launch_bounds__(256) void wgrad_batch_fold_kernel(WgradBatch w) {
     float *out = w.dw[t.job];
     const int ld = w.lddw[t.job];
     const float *first = w.pieces + size_t(piece_slot(w, tile, 0)) * (BM * BN);
-    constexpr int QUADS = BN / 4, ROWS = BM / 4;
-    for (int i = threadIdx.x; i < ROWS * QUADS; i += 256) {
+    constexpr int QUADS = BN / 4, ROWS = BM / 4, PER_THREAD = ROWS * QUADS / 256;
+    static_assert(ROWS * QUADS % 256 == 0, "a quarter tile is a whole number of float4 per thread");
+    const auto finish = [&](int i, float4 sum) {
         const int r = part * ROWS + i / QUADS, c = (i % QUADS) * 4;
-        float4 sum = make_float4(0, 0, 0, 0);
-        for (int split = 0; split < splits; ++split) { // fixed order
-            const float4 v = *reinterpret_cast<const float4 *>(first + size_t(split) * (BM * BN) + r * BN + c);
-            sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
-        }
         float4 *p = reinterpret_cast<float4 *>(out + size_t(t.m0 + r) * ld + t.n0 + c);
         if (w.accumulate) {
             const float4 old = *p;
             sum.x += old.x, sum.y += old.y, sum.z += old.z, sum.w += old.w;
         }
         *p = sum;
+    };
+    const float *mine = first + size_t(part) * ROWS * BN + threadIdx.x * 4; // a quarter tile is contiguous
+    if (splits == 2) { // most tiles: every load of the thread is requested before the first sum
+        float4 a[PER_THREAD], b[PER_THREAD];
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k) {
+            a[k] = *reinterpret_cast<const float4 *>(mine + k * 1024);
+            b[k] = *reinterpret_cast<const float4 *>(mine + k * 1024 + BM * BN);
+        }
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k)
+            finish(threadIdx.x + k * 256, make_float4(a[k].x + b[k].x, a[k].y + b[k].y, a[k].z + b[k].z, a[k].w + b[k].w));
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < PER_THREAD; ++k) {
+        float4 sum = make_float4(0, 0, 0, 0);
+#pragma unroll 4
+        for (int split = 0; split < splits; ++split) { // fixed order
+            const float4 v = *reinterpret_cast<const float4 *>(mine + k * 1024 + size_t(split) * (BM * BN));
+            sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+        }
+        finish(threadIdx.x + k * 256, sum);
     }
 }
 
