@@ -90,8 +90,8 @@ def zipf_bytes(n, rng, s=1.1):
     return np.minimum(np.searchsorted(cdf, rng.random(n)), 255).astype(np.uint8)
 
 
-def cpu_baseline(sequences=4):
-    """The CPU checker on 4 of the step's 16 sequences (same model, B=4): forward, backward, AdamW."""
+def cpu_baseline(sequences=8):
+    """The CPU checker on 8 of the step's 16 sequences (same model, B=8): forward, backward, AdamW."""
     import oracle
     cfg = oracle.model(depth=L, context=T, batch=sequences, d_model=D, heads=H)
     w = oracle.init_weights(cfg)
