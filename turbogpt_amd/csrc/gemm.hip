@@ -69,6 +69,10 @@ struct EpilogueBf16 {
             for (int e = 0; e < 4; ++e)
                 g[e] = pack_bf16(gelu_f(bf16_lo(y[e])), gelu_f(bf16_hi(y[e])));
             *reinterpret_cast<u32x4 *>(out2 + size_t(m) * ld_out2 + n) = g;
+            // the pre-activation is not read again before the backward pass: kept out of the caches' way, the
+            // activation next to it stays there for the projection that follows (measured -0.8 % on the step)
+            __builtin_nontemporal_store(y, reinterpret_cast<u32x4 *>(out + size_t(m) * ld_out + n));
+            return;
         }
         *reinterpret_cast<u32x4 *>(out + size_t(m) * ld_out + n) = y;
     }
