@@ -480,6 +480,8 @@ __global__ __launch_bounds__(256) void adamw_kernel(bf16_t *__restrict__ hi, uin
         __syncthreads();
         scale = clip_scale;
     }
+    // Every stream here is touched once per step: non-temporal loads and stores keep 3 GB of optimizer state from
+    // evicting what the next step's first kernels read (measured -0.6 % on the step).
     const size_t quads = n >> 2;
     for (size_t q = blockIdx.x * size_t(256) + threadIdx.x; q < quads; q += size_t(gridDim.x) * 256) {
         const size_t i = q * 4;
@@ -494,9 +496,9 @@ __global__ __launch_bounds__(256) void adamw_kernel(bf16_t *__restrict__ hi, uin
         if (flags[lo_s] & 2) // owned by another optimizer (Muon, cuda/optim.cuh:94-96)
             continue;
         const float decay = (flags[lo_s] & 1) ? a.weight_decay : 0.f;
-        const f32x4 gv = *reinterpret_cast<const f32x4 *>(g + i);
-        f32x4 mv = *reinterpret_cast<const f32x4 *>(m + i), vv = *reinterpret_cast<const f32x4 *>(v + i);
-        const u32x2 hv = *reinterpret_cast<const u32x2 *>(hi + i), lv = *reinterpret_cast<const u32x2 *>(lo + i);
+        const f32x4 gv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(g + i));
+        f32x4 mv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(m + i)), vv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(v + i));
+        const u32x2 hv = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(hi + i)), lv = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(lo + i));
         uint32_t bits[4] = {(hv.x << 16) | (lv.x & 0xffffu), (hv.x & 0xffff0000u) | (lv.x >> 16),
                             (hv.y << 16) | (lv.y & 0xffffu), (hv.y & 0xffff0000u) | (lv.y >> 16)};
 #pragma unroll
@@ -509,15 +511,15 @@ __global__ __launch_bounds__(256) void adamw_kernel(bf16_t *__restrict__ hi, uin
             const float w = __uint_as_float(bits[k]) * (1.f - a.lr * decay);
             bits[k] = __float_as_uint(w - (a.lr / a.bc1) * mk / (sqrtf(vk) / a.sqrt_bc2 + a.eps));
         }
-        *reinterpret_cast<f32x4 *>(m + i) = mv;
-        *reinterpret_cast<f32x4 *>(v + i) = vv;
+        __builtin_nontemporal_store(mv, reinterpret_cast<f32x4 *>(m + i));
+        __builtin_nontemporal_store(vv, reinterpret_cast<f32x4 *>(v + i));
         u32x2 ho, lw;
         ho.x = (bits[0] >> 16) | (bits[1] & 0xffff0000u);
         ho.y = (bits[2] >> 16) | (bits[3] & 0xffff0000u);
         lw.x = (bits[0] & 0xffffu) | (bits[1] << 16);
         lw.y = (bits[2] & 0xffffu) | (bits[3] << 16);
-        *reinterpret_cast<u32x2 *>(hi + i) = ho;
-        *reinterpret_cast<u32x2 *>(lo + i) = lw;
+        __builtin_nontemporal_store(ho, reinterpret_cast<u32x2 *>(hi + i));
+        __builtin_nontemporal_store(lw, reinterpret_cast<u32x2 *>(lo + i));
     }
 }
 
@@ -592,7 +594,7 @@ __global__ __launch_bounds__(256) void transpose_batch_kernel(const bf16_t *__re
     for (int i = 0; i < 8; ++i) {
         const int c = ty + i * 8; // source column = destination row
         const uint32_t pair = uint32_t(tile[tx * 2][c]) | (uint32_t(tile[tx * 2 + 1][c]) << 16);
-        *reinterpret_cast<uint32_t *>(dst + size_t(c0 + c) * job.rows + r0 + tx * 2) = pair;
+        __builtin_nontemporal_store(pair, reinterpret_cast<uint32_t *>(dst + size_t(c0 + c) * job.rows + r0 + tx * 2));
     }
 }
 

@@ -798,7 +798,7 @@ __global__ __launch_bounds__(256) void wgrad_batch_fold_kernel(WgradBatch w) {
             const float4 old = *p;
             sum.x += old.x, sum.y += old.y, sum.z += old.z, sum.w += old.w;
         }
-        *p = sum;
+        __builtin_nontemporal_store(f32x4{sum.x, sum.y, sum.z, sum.w}, reinterpret_cast<f32x4 *>(p));
     };
     const float *mine = first + size_t(part) * ROWS * BN + threadIdx.x * 4; // a quarter tile is contiguous
     if (splits == 2) { // most tiles: every load of the thread is requested before the first sum
@@ -845,7 +845,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
             const float4 old = *p;
             sum.x += old.x, sum.y += old.y, sum.z += old.z, sum.w += old.w;
         }
-        *p = sum;
+        __builtin_nontemporal_store(f32x4{sum.x, sum.y, sum.z, sum.w}, reinterpret_cast<f32x4 *>(p));
     }
 }
 
