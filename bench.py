@@ -28,7 +28,7 @@ M = B * T
 ALGORITHMIC_BYTES_PER_LAUNCH = sum(2 * (M * k + n * k + M * n) for n, k in
                                    [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
 # HBM bytes per launch of that kernel, measured with rocprofv3 FETCH_SIZE / WRITE_SIZE runs of --traffic-probe
-HBM_TRAFFIC_PER_LAUNCH = 150.3e6
+HBM_TRAFFIC_PER_LAUNCH = 151.0e6
 
 
 def gemm_flops():
