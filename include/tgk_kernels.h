@@ -111,6 +111,18 @@ TGK_API int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, const 
                          const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ, uint16_t *dK,
                          uint16_t *dV, int lddq, float scale, void *workspace, size_t workspace_bytes);
 TGK_API size_t tgk_attn_bwd_workspace(int B, int H, int T);
+/* tgk_attn_bwd without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * two row vectors the backward kernels exchange (2 * B*H*T floats) live in a device array inside the library:
+ * 8 MiB per GPU the library runs on, held until the process ends.  B*H*T <= tgk_attn_bwd_static_max_rows()
+ * (1048576); larger shapes are rejected and need tgk_attn_bwd.  The call allocates and frees nothing.  All
+ * calls on one GPU share the array: calls that overlap on one GPU (different streams or threads) race.
+ * Same kernels and results, bit for bit, as tgk_attn_bwd. */
+TGK_API int tgk_attn_bwd_static(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
+                                const uint16_t *K, const uint16_t *V, int ld, const uint16_t *O, int ldo,
+                                const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ, uint16_t *dK,
+                                uint16_t *dV, int lddq, float scale);
+TGK_API size_t tgk_attn_bwd_static_max_rows(void);
 
 /* ---- HBM-bound operators.  Parameters are held as two 16-bit halves of their fp32 master:
  * `hi` (the bf16 compute weight, truncated) and `lo` (cuda/ops.cuh:6-14); operators that need

@@ -29,6 +29,9 @@ KERNEL_ABI = {
     "tgk_attn_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32,
                            f32, vp, sz]),
     "tgk_attn_bwd_workspace": (sz, [i32, i32, i32]),
+    "tgk_attn_bwd_static": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32,
+                                  f32]),
+    "tgk_attn_bwd_static_max_rows": (sz, []),
     "tgk_embed_fwd": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
     "tgk_embed_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32, vp, sz]),
     "tgk_embed_bwd_workspace": (sz, [i32, i32]),

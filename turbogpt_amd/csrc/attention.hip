@@ -16,6 +16,7 @@
 // tiles).  No atomics: every output element has one owner and a fixed summation order, so results
 // are bit-reproducible.
 #include "common.h"
+#include <atomic>
 #include "../../include/tgk_kernels.h"
 
 namespace {
@@ -599,31 +600,90 @@ extern "C" size_t tgk_attn_bwd_workspace(int B, int H, int T) {
     return 2 * size_t(B) * H * T * sizeof(float); // delta, and the log-sum-exp in base 2
 }
 
+namespace {
+void attn_bwd_check(int B, int H, int T, int hd, const uint16_t *Q, const uint16_t *K, const uint16_t *V, int ld,
+                    const uint16_t *O, int ldo, const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ,
+                    uint16_t *dK, uint16_t *dV, int lddq) {
+    check_attention_shape(B, H, T, hd);
+    check_matrix(Q, ld, "Q");
+    check_matrix(K, ld, "K");
+    check_matrix(V, ld, "V");
+    check_matrix(O, ldo, "O");
+    check_matrix(dO, lddo, "dO");
+    check_matrix(dQ, lddq, "dQ");
+    check_matrix(dK, lddq, "dK");
+    check_matrix(dV, lddq, "dV");
+    require(lse && !(reinterpret_cast<uintptr_t>(lse) & 15), "attention: lse must be 16-byte aligned");
+}
+// both backward kernels; `rows` holds delta[B*H*T] followed by the base-2 log-sum-exps[B*H*T]
+void attn_bwd_launch(hipStream_t stream, int B, int H, int T, const uint16_t *Q, const uint16_t *K,
+                     const uint16_t *V, int ld, const uint16_t *O, int ldo, const float *lse, const uint16_t *dO,
+                     int lddo, uint16_t *dQ, uint16_t *dK, uint16_t *dV, int lddq, float scale, float *rows) {
+    float *delta = rows, *lse2 = delta + size_t(B) * H * T;
+    const dim3 grid(causal_grid(T / 128, B * H));
+    hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, O, ldo, lse, lse2,
+                       delta, dQ, lddq, T, H, B * H, scale);
+    hipLaunchKernelGGL(attn_bwd_dkdv_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse2, delta, dK, dV,
+                       lddq, T, H, B * H, scale);
+    check_hip(hipGetLastError(), "attention backward launch: ");
+}
+} // namespace
+
 extern "C" int tgk_attn_bwd(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
                             const uint16_t *K, const uint16_t *V, int ld, const uint16_t *O, int ldo,
                             const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ, uint16_t *dK,
                             uint16_t *dV, int lddq, float scale, void *workspace,
                             size_t workspace_bytes) {
     return guarded([&] {
-        check_attention_shape(B, H, T, hd);
-        check_matrix(Q, ld, "Q");
-        check_matrix(K, ld, "K");
-        check_matrix(V, ld, "V");
-        check_matrix(O, ldo, "O");
-        check_matrix(dO, lddo, "dO");
-        check_matrix(dQ, lddq, "dQ");
-        check_matrix(dK, lddq, "dK");
-        check_matrix(dV, lddq, "dV");
-        require(lse && !(reinterpret_cast<uintptr_t>(lse) & 15), "attention: lse must be 16-byte aligned");
+        attn_bwd_check(B, H, T, hd, Q, K, V, ld, O, ldo, lse, dO, lddo, dQ, dK, dV, lddq);
         require(workspace && workspace_bytes >= tgk_attn_bwd_workspace(B, H, T) &&
                     !(reinterpret_cast<uintptr_t>(workspace) & 15),
                 "attention backward: workspace too small (see tgk_attn_bwd_workspace)");
-        float *delta = static_cast<float *>(workspace), *lse2 = delta + size_t(B) * H * T;
-        const dim3 grid(causal_grid(T / 128, B * H));
-        hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, O, ldo, lse,
-                           lse2, delta, dQ, lddq, T, H, B * H, scale);
-        hipLaunchKernelGGL(attn_bwd_dkdv_kernel, grid, dim3(256), 0, stream, Q, K, V, ld, dO, lddo, lse2, delta,
-                           dK, dV, lddq, T, H, B * H, scale);
-        check_hip(hipGetLastError(), "attention backward launch: ");
+        attn_bwd_launch(stream, B, H, T, Q, K, V, ld, O, ldo, lse, dO, lddo, dQ, dK, dV, lddq, scale,
+                        static_cast<float *>(workspace));
+    });
+}
+
+// ---- the same backward for callers that cannot allocate -------------------------------------------
+// The two row vectors the kernels exchange (delta and the base-2 log-sum-exp, B*H*T floats each) live in
+// a device array of this library instead of a caller's workspace.  Every GPU the library runs on holds
+// its own copy of the array at its own address; the address is looked up once per device, with that
+// device current, and only that address - never the array's name - is handed to kernels.  The dQ kernel
+// overwrites every row the dK/dV kernel reads, so nothing has to be cleared between calls.
+namespace {
+constexpr size_t STATIC_BWD_ROWS = size_t(1) << 20; // B*H*T of one call: 8 MiB of device memory per GPU
+static __device__ __align__(256) float scratch[2 * STATIC_BWD_ROWS];
+constexpr int STATIC_MAX_DEVICES = 64;
+std::atomic<float *> scratch_address[STATIC_MAX_DEVICES];
+
+float *scratch_on_current_device() {
+    int device = 0;
+    check_hip(hipGetDevice(&device), "attention backward (static): ");
+    require(device >= 0 && device < STATIC_MAX_DEVICES, "attention backward (static): device index out of range");
+    float *address = scratch_address[device].load(std::memory_order_acquire);
+    if (!address) {
+        void *found = nullptr;
+        check_hip(hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)), "attention backward (static) scratch address: ");
+        require(found != nullptr, "attention backward (static): the scratch array has no device address");
+        address = static_cast<float *>(found);
+        scratch_address[device].store(address, std::memory_order_release);
+    }
+    return address;
+}
+} // namespace
+
+extern "C" size_t tgk_attn_bwd_static_max_rows(void) { return STATIC_BWD_ROWS; }
+
+extern "C" int tgk_attn_bwd_static(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
+                                   const uint16_t *K, const uint16_t *V, int ld, const uint16_t *O, int ldo,
+                                   const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ, uint16_t *dK,
+                                   uint16_t *dV, int lddq, float scale) {
+    return guarded([&] {
+        attn_bwd_check(B, H, T, hd, Q, K, V, ld, O, ldo, lse, dO, lddo, dQ, dK, dV, lddq);
+        require(size_t(B) * H * T <= STATIC_BWD_ROWS,
+                "attention backward (static): B*H*T exceeds tgk_attn_bwd_static_max_rows() = 1048576; "
+                "use tgk_attn_bwd with a workspace");
+        attn_bwd_launch(stream, B, H, T, Q, K, V, ld, O, ldo, lse, dO, lddo, dQ, dK, dV, lddq, scale,
+                        scratch_on_current_device());
     });
 }
