@@ -147,11 +147,18 @@ def kernel_sweeps(out):
             "wgrad": lambda: check(lib.tgk_gemm_wgrad(stream, M, n, k, dy.data_ptr(), n, x.data_ptr(), k,
                                                       dw.data_ptr(), k, 0, ws.data_ptr(), need)),
         }
+        # comparator only, never in the product: the vendor library (hipBLASLt behind torch.matmul) on the same
+        # operands - forward X W^T, dgrad dY W, wgrad dY^T X (bf16 out where ours is fp32)
+        library_runs = {"fwd": lambda: torch.matmul(x, w.t(), out=y), "dgrad": lambda: torch.matmul(dy, w, out=dx),
+                        "wgrad": lambda: torch.matmul(dy.t(), x)}
+        library_ms = {name: timed(fn) for name, fn in library_runs.items()}
         for name, fn in runs.items():
             ms = timed(fn)
+            versus = library_ms.get(name.replace("_t", ""))
             print(json.dumps({"kernel": f"gemm_{name}", "M": M, "K": k, "N": n, "ms": round(ms, 4),
                               "tflops": round(flop / ms / 1e9, 1),
-                              "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
+                              "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                              "vendor_library_tflops": round(flop / versus / 1e9, 1)}), file=out)
     # the four weight gradients of one block in one launch, as the engine runs them
     import ctypes
     from turbogpt_amd.bridge import WgradJob
