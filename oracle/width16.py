@@ -13,8 +13,9 @@ one radian per position), causal arg-max attention with a GELU gate, SwiGLU(48),
 ``exact=True`` runs the same graph in float64 without any rounding or weight truncation; that variant
 is what finite differences pin, and the rounded variant is checked against it.
 
-What pins it (tests/test_oracle_width16.py): finite differences of the float64 variant for every
-parameter tensor; rounded against float64 within bf16 resolution; the RoPE table against
+What pins it (tests/test_oracle_width16.py): the float64 variant against the same network assembled only from
+torch library ops and autograd (tests/torch_width16.py: logits 1e-9, every gradient tensor 1e-6); finite
+differences of the float64 variant for every parameter tensor; rounded against float64 within bf16 resolution; the RoPE table against
 float32(cos k), float32(sin k) and the eight constants of cuda/attention.cuh:7-14; the tie rule
 (first key wins); causality; the AdamW part against torch.optim.AdamW and the Muon part against
 torch.optim.Muon (library routines); the 64-small-steps known answer of tests/verify.py:108-127.

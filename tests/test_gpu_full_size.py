@@ -86,3 +86,37 @@ def test_training_is_deterministic_and_learns_at_full_size(name):
     assert np.isfinite(per_step).all()
     assert abs(per_step[0] - np.log(256)) < 0.6
     assert per_step[-1] < per_step[0] - 0.02  # six AdamW steps already lower the loss
+
+
+def test_headline_shape_against_the_checker(orc):
+    """One sequence of the headline model (d768 L12 H12 T1024, the shape bench.py times at batch 16) through
+    tg_batch against the CPU checker on the same weights and tokens: logits and the flat gradient to 1e-2,
+    every parameter tensor's gradient to 2e-2, mean loss to 3e-3 (tests/verify.py:31-42 of the reference)."""
+    cfg = dict(CONFIGS["configs[3]"], batch=1)
+    T, d = cfg["context"], cfg["d_model"]
+    oc = orc.model(cfg["depth"], T, 1, d, cfg["heads"])
+    with Native(ModelConfig(**cfg)) as engine:
+        assert engine.count == orc.parameter_count(oc)
+        w = weights(engine.count, cfg, 3407)
+        rng = np.random.default_rng(5)
+        for name, offset, shape in orc.Layout(oc).entries:  # norm parameters off their defaults
+            if name.endswith(("_g", "_b")):
+                w[offset:offset + shape[0]] += rng.standard_normal(shape[0]).astype(np.float32) * 0.1
+        engine.set_weights(w)
+        x = zipf_bytes(T, 71).reshape(1, T)
+        y = np.roll(x, -1, axis=1)
+        logits, grad, losses = engine.batch(x, y)
+    want_logits, want_grad, want_loss = orc.model_batch(oc, w, x, y)
+
+    def rel(a, b):
+        a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+        return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-12))
+
+    assert rel(logits, want_logits) < 1e-2
+    assert abs(float(losses.mean()) - float(want_loss.mean())) < 3e-3
+    assert rel(grad, want_grad) < 1e-2
+    worst = max((rel(grad[o:o + int(np.prod(s))], want_grad[o:o + int(np.prod(s))]), name)
+                for name, o, s in orc.Layout(oc).entries)
+    print(f"headline shape: logits {rel(logits, want_logits):.3g}, gradient {rel(grad, want_grad):.3g}, worst tensor {worst}",
+          flush=True)
+    assert worst[0] < 2e-2, worst

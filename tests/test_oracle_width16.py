@@ -48,6 +48,28 @@ def test_rope_table_is_the_reference_constant_table():
     np.testing.assert_array_equal(sin, np.array(sin_ref, dtype=np.float32))
 
 
+@pytest.mark.parametrize("depth,context,batch,seed", [(4, 8, 6, 11), (8, 4, 5, 12), (4, 4, 16, 13)])
+def test_float64_model_equals_a_model_of_torch_library_ops(depth, context, batch, seed):
+    """The float64 variant of the checker against the same network assembled only from torch library ops
+    (tests/torch_width16.py) and differentiated by autograd: logits to 1e-9, every parameter tensor's
+    gradient to 1e-6, per-position losses to 1e-9.  A wrong RoPE pairing, a wrong gate (gelu of the winning
+    score), SiLU in the place of the up projection or a wrong head layout fails here; the rounded variant is
+    tied to this one by test_rounded_model_tracks_the_exact_one."""
+    import torch_width16
+    rng = np.random.default_rng(seed)
+    flat = random_weights(depth, seed).astype(np.float64)
+    x = rng.integers(0, 256, (batch, context), dtype=np.uint8)
+    y = rng.integers(0, 256, (batch, context), dtype=np.uint8)
+    model = w16.Width16(depth, context, batch, exact=True)
+    logits, grad, position_losses = model.batch(flat, x, y)
+    want_logits, want_grad, want_losses = torch_width16.forward_backward(model.entries, flat, x, y, depth)
+    assert relative(logits, want_logits) < 1e-9
+    np.testing.assert_allclose(position_losses, want_losses.mean(0), rtol=0, atol=1e-9)
+    for name, (offset, shape) in model.entries.items():
+        n = int(np.prod(shape))
+        assert relative(grad[offset:offset + n], want_grad[offset:offset + n]) < 1e-6, name
+
+
 def test_rounding_helpers():
     x = np.array([1.0, 1.00390625, 1.005859375, 3.14159265, -2.71828], np.float32)
     # 1 + 2^-8 is a tie between 1.0 and 1 + 2^-7: nearest even keeps 1.0; 1 + 3*2^-9 rounds up
