@@ -205,6 +205,31 @@ def test_resume_from_a_checkpoint_file(orc, tmp_path):
         b.close()
 
 
+# the keys of the reference's JSON lines, in its order: report.cpp:46-59, :61-80, :82-117
+CONFIG_KEYS = ["architecture", "depth", "ctx", "batch", "inflight", "chunk", "optimizer", "parameters", "blocks",
+               "shared_bytes", "steps", "dataset_bytes", "schedule", "warmup_fraction", "initial_lr_fraction",
+               "final_lr_fraction", "low_momentum", "high_momentum"]
+STEP_KEYS = ["step", "tokens", "last_bpb", "position_bpb", "adam_lr", "muon_lr", "momentum", "train_seconds",
+             "tokens_per_second"]
+SUMMARY_KEYS = ["architecture", "depth", "ctx", "batch", "inflight", "chunk", "seed", "optimizer", "learning_rate", "muon_lr",
+                "schedule", "schedule_steps", "warmup_fraction", "initial_lr_fraction", "final_lr_fraction", "low_momentum",
+                "high_momentum", "requested_tokens", "tokens", "final_loss", "final_bpb", "position_bpb", "sample",
+                "initialization_seconds", "mean_staleness", "max_staleness", "dataset_load_seconds", "training_seconds",
+                "sample_seconds", "process_seconds", "tokens_per_second", "sample_temperature"]
+
+
+def host_program_lines(stdout):
+    """-> (config object, step objects, summary object); asserts the reference's keys lead every object in order."""
+    import json
+    lines = [json.loads(line) for line in stdout.splitlines()]
+    config, steps, summary = lines[0]["config"], lines[1:-1], lines[-1]["summary"]
+    assert list(config)[:len(CONFIG_KEYS)] == CONFIG_KEYS
+    for step in steps:
+        assert list(step)[:len(STEP_KEYS)] == STEP_KEYS
+    assert list(summary)[:len(SUMMARY_KEYS)] == SUMMARY_KEYS
+    return config, steps, summary
+
+
 def test_host_program_trains_and_resumes(orc, tmp_path):
     """turbogpt_amd/host/train_bytes (plain g++ over the C ABI): the loss falls; 12 steps in one run equal
     6 steps + checkpoint + 6 resumed steps, to the last printed digit (trainer.cpp:51-80,105-121)."""
@@ -221,17 +246,23 @@ def test_host_program_trains_and_resumes(orc, tmp_path):
     def run(*extra):
         done = subprocess.run(common + list(extra), capture_output=True, text=True, timeout=120)
         assert done.returncode == 0, done.stderr
-        return [json.loads(line) for line in done.stdout.splitlines()]
+        return host_program_lines(done.stdout)
 
-    whole = run("--save", str(tmp_path / "whole.pt"))
-    assert [r["step"] for r in whole[:-1]] == [3, 6, 9, 12] and whole[-1]["steps"] == 12
-    assert whole[-2]["loss"] < whole[0]["loss"] - 0.05 and len(whole[-1]["sample"]) == 68
+    config, chunks, whole = run("--save", str(tmp_path / "whole.pt"))
+    assert config["architecture"] == "gelu-layernorm-softmax" and config["optimizer"] == "adamw" and config["steps"] == 12
+    assert config["d_model"] == 128 and config["ctx"] == 128 and config["dataset_bytes"] == 1 << 16
+    assert [r["step"] for r in chunks] == [3, 6, 9, 12] and whole["steps"] == 12
+    assert [r["tokens"] for r in chunks] == [n * 4 * 128 for n in (3, 6, 9, 12)]
+    assert all(len(r["position_bpb"]) == 128 and r["last_bpb"] == r["position_bpb"][-1] for r in chunks)
+    assert chunks[-1]["loss"] < chunks[0]["loss"] - 0.05 and len(whole["sample"]) == 68
+    assert whole["tokens_per_second"] > 0 and whole["sample_temperature"] == 1.0
     # a run cut after six steps: same schedule (--tokens), fewer steps trained
     first = subprocess.run(common + ["--save", str(tmp_path / "half.pt"), "--chunk", "6"], capture_output=True, text=True,
                            timeout=120, env={"TRAIN_BYTES_STOP_AFTER": "6", **__import__("os").environ})
     assert first.returncode == 0, first.stderr
-    resumed = run("--load", str(tmp_path / "half.pt"), "--save", str(tmp_path / "resumed.pt"))
-    assert resumed[-1]["steps"] == 12 and resumed[-1]["final_loss"] == whole[-1]["final_loss"]
+    _, _, resumed = run("--load", str(tmp_path / "half.pt"), "--save", str(tmp_path / "resumed.pt"))
+    assert resumed["steps"] == 12 and resumed["final_loss"] == whole["final_loss"] and resumed["last_loss"] == whole["last_loss"]
+    assert resumed["position_bpb"] == whole["position_bpb"]
     from turbogpt_amd.bridge import read_checkpoint
     a, b = read_checkpoint(tmp_path / "whole.pt"), read_checkpoint(tmp_path / "resumed.pt")
     np.testing.assert_array_equal(a["weights"].view(np.uint32), b["weights"].view(np.uint32))
@@ -256,10 +287,14 @@ def test_host_program_logs_a_run(orc, tmp_path):
                            "--inflight", "4", "--log-to", str(run_dir), "--save", str(tmp_path / "w16.pt")],
                           capture_output=True, text=True, timeout=120)
     assert done.returncode == 0, done.stderr
-    lines = [json.loads(line) for line in done.stdout.splitlines()]
-    assert [r["step"] for r in lines[:-1]] == [50, 100, 150, 200, 250, 300]
-    assert lines[-2]["loss"] < lines[0]["loss"] - 0.3  # it learns the Zipf byte frequencies
+    config, lines, summary = host_program_lines(done.stdout)
+    assert config["architecture"] == "swiglu48-rmsnorm-rope" and config["optimizer"] == "muon" and config["parameters"] == 21648
+    assert [r["step"] for r in lines] == [50, 100, 150, 200, 250, 300]
+    assert lines[-1]["loss"] < lines[0]["loss"] - 0.3  # it learns the Zipf byte frequencies
+    assert lines[-1]["muon_lr"] < lines[1]["muon_lr"] and lines[-1]["adam_lr"] < lines[1]["adam_lr"]  # OneCycle descends
     report = json.loads((run_dir / "report.json").read_text())
+    assert report == summary and list(report)[:len(SUMMARY_KEYS)] == SUMMARY_KEYS  # the file holds the summary object
+    assert report["tokens_per_second"] > 0  # also with --save and --log-to together
     assert report["architecture"] == "swiglu48-rmsnorm-rope" and report["optimizer"] == "muon"
     assert report["parameters"] == 21648 and report["steps"] == steps and report["tokens"] == steps * batch * context
     assert report["final_loss_batches"] == 3 and len(report["position_bpb"]) == context  # last ceil(300 / 100) steps
@@ -276,7 +311,7 @@ def test_host_program_logs_a_run(orc, tmp_path):
         if one(tensor, 1) == 1:
             scalars.setdefault(one(value, 1).decode(), []).append((one(event, 2), struct.unpack("<f", one(tensor, 5))[0]))
     assert [step for step, _ in scalars["loss"]] == [n * batch * context for n in (50, 100, 150, 200, 250, 300)]
-    assert scalars["loss"][-1][1] == pytest.approx(lines[-2]["loss"], abs=1e-5)
+    assert scalars["loss"][-1][1] == pytest.approx(lines[-1]["loss"], abs=1e-5)
     assert scalars["bits-per-byte"][-1][1] == pytest.approx(scalars["last_loss"][-1][1] / np.log(2), rel=1e-6)
     assert scalars["model_bytes"] == [(0, 21648 * 4.0)] and scalars["lr"][-1][1] < scalars["lr"][1][1]
     from turbogpt_amd.bridge import read_checkpoint

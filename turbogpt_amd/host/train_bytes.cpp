@@ -7,9 +7,12 @@
 //   - checkpoint at the end, resume with --load (trainer.cpp:51-55,76-80,105-121)
 //   - a top-10 sample from the trained model (sampling.cpp:10-42)
 //   - --log-to DIR: TensorBoard events per chunk (training_log.cpp:55-97) and DIR/report.json with the loss
-//     averaged over the last 1 % of the steps (loss_summary.cpp:5-29, report.cpp:83-131)
+//     averaged over the last 1 % of the steps (loss_summary.cpp:5-29, report.cpp:82-131)
 //   - --width16 1: the reference's own network through tg_create (depth 4/8, context 4/8)
-// Prints one JSON line per chunk and a final one.
+// Standard output carries the reference's JSON lines, key for key and in its order: {"config":{...}} once
+// (report.cpp:46-59), one {"step":...} object per chunk (report.cpp:61-80) and {"summary":{...}} at the end
+// (report.cpp:82-117); keys the reference does not have (d_model, heads, ffn, vocab, loss, steps, parameters,
+// final_loss_batches, last_loss) follow the reference's inside each object.
 #include "tg_checkpoint.h"
 #include "tg_events.h"
 #include "tg_model.h"
@@ -23,7 +26,9 @@
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <iomanip>
 #include <iostream>
+#include <sstream>
 #include <numeric>
 #include <random>
 #include <stdexcept>
@@ -160,6 +165,98 @@ double seconds_since(std::chrono::steady_clock::time_point start) {
     return std::chrono::duration<double>(std::chrono::steady_clock::now() - start).count();
 }
 
+// a JSON string literal: control characters and bytes beyond ASCII as \u00XX (report.cpp:9-43)
+void json_string(std::ostream &out, const std::string &value) {
+    static const char hex[] = "0123456789abcdef";
+    out << '"';
+    for (unsigned char byte : value) {
+        if (byte == '"' || byte == '\\')
+            out << '\\' << char(byte);
+        else if (byte == '\n')
+            out << "\\n";
+        else if (byte == '\r')
+            out << "\\r";
+        else if (byte == '\t')
+            out << "\\t";
+        else if (byte < 0x20 || byte >= 0x80)
+            out << "\\u00" << hex[byte >> 4] << hex[byte & 15];
+        else
+            out << char(byte);
+    }
+    out << '"';
+}
+const char *architecture(const Options &o) { return o.width16 ? "swiglu48-rmsnorm-rope" : "gelu-layernorm-softmax"; }
+const char *optimizer(const Options &o) { return o.width16 ? "muon" : "adamw"; }
+
+// {"config":{...}}: the keys of report.cpp:46-59 in its order, then the model shape the reference has no field for
+void log_config(Engine *engine, const Options &o, const OneCycle &schedule, int steps, int64_t dataset_bytes) {
+    const TgModelConfig &m = o.model;
+    std::cout << "{\"config\":{\"architecture\":\"" << architecture(o) << "\",\"depth\":" << m.base.depth
+              << ",\"ctx\":" << m.base.context << ",\"batch\":" << m.base.batch << ",\"inflight\":" << m.base.inflight
+              << ",\"chunk\":" << o.chunk << ",\"optimizer\":\"" << optimizer(o)
+              << "\",\"parameters\":" << tg_parameter_count(engine) << ",\"blocks\":" << tg_blocks(engine)
+              << ",\"shared_bytes\":" << tg_shared_bytes(engine) << ",\"steps\":" << steps
+              << ",\"dataset_bytes\":" << dataset_bytes << ",\"schedule\":\"onecycle\""
+              << ",\"warmup_fraction\":" << schedule.warmup_fraction
+              << ",\"initial_lr_fraction\":" << schedule.initial_lr_fraction
+              << ",\"final_lr_fraction\":" << schedule.final_lr_fraction << ",\"low_momentum\":" << schedule.low_momentum
+              << ",\"high_momentum\":" << schedule.high_momentum << ",\"d_model\":" << m.d_model
+              << ",\"heads\":" << m.heads << ",\"ffn\":" << m.ffn << ",\"vocab\":" << m.vocab << "}}" << std::endl;
+}
+
+// one object per chunk: report.cpp:61-80 (losses of the chunk's last step, cumulative time and rate), then "loss"
+void log_step(const Options &o, const OneCycle &schedule, const float *losses, int done, double train_seconds) {
+    const TgModelConfig &m = o.model;
+    const int64_t per_step = int64_t(m.base.batch) * m.base.context;
+    const double log2 = std::log(2.0);
+    std::cout << "{\"step\":" << done << ",\"tokens\":" << done * per_step
+              << ",\"last_bpb\":" << losses[m.base.context - 1] / log2 << ",\"position_bpb\":[";
+    for (int position = 0; position < m.base.context; ++position)
+        std::cout << (position ? "," : "") << losses[position] / log2;
+    StepRates rates{};
+    check(tg_onecycle_point(&schedule, done - 1, &rates));
+    std::cout << "],\"adam_lr\":" << m.base.learning_rate * rates.multiplier
+              << ",\"muon_lr\":" << m.base.muon_lr * rates.multiplier << ",\"momentum\":" << rates.momentum
+              << ",\"train_seconds\":" << train_seconds << ",\"tokens_per_second\":" << done * per_step / train_seconds
+              << ",\"loss\":" << std::accumulate(losses, losses + m.base.context, 0.0) / m.base.context << "}" << std::endl;
+}
+
+struct RunReport {
+    int steps, done;
+    std::vector<double> final_losses; // per position, averaged over the last 1 % of the steps
+    uint64_t final_loss_batches;
+    std::string sample;
+    double initialize_seconds, load_seconds, train_seconds, sample_seconds, total, mean_staleness, last_loss;
+    int max_staleness;
+    int64_t parameters;
+};
+// the summary object: report.cpp:82-117 key for key, then the added keys
+void report(std::ostream &out, const Options &o, const OneCycle &schedule, const RunReport &r) {
+    const TgModelConfig &m = o.model;
+    const double log2 = std::log(2.0), final_loss = r.final_losses.back();
+    const int64_t tokens = r.steps * (int64_t(m.base.batch) * m.base.context);
+    out << std::setprecision(10) << "{\"architecture\":\"" << architecture(o) << "\",\"depth\":" << m.base.depth
+        << ",\"ctx\":" << m.base.context << ",\"batch\":" << m.base.batch << ",\"inflight\":" << m.base.inflight
+        << ",\"chunk\":" << o.chunk << ",\"seed\":" << m.base.seed << ",\"optimizer\":\"" << optimizer(o)
+        << "\",\"learning_rate\":" << m.base.learning_rate << ",\"muon_lr\":" << m.base.muon_lr
+        << ",\"schedule\":\"onecycle\",\"schedule_steps\":" << r.steps
+        << ",\"warmup_fraction\":" << schedule.warmup_fraction << ",\"initial_lr_fraction\":" << schedule.initial_lr_fraction
+        << ",\"final_lr_fraction\":" << schedule.final_lr_fraction << ",\"low_momentum\":" << schedule.low_momentum
+        << ",\"high_momentum\":" << schedule.high_momentum << ",\"requested_tokens\":" << o.tokens << ",\"tokens\":" << tokens
+        << ",\"final_loss\":" << final_loss << ",\"final_bpb\":" << final_loss / log2 << ",\"position_bpb\":[";
+    for (size_t position = 0; position < r.final_losses.size(); ++position)
+        out << (position ? "," : "") << r.final_losses[position] / log2;
+    out << "],\"sample\":";
+    json_string(out, r.sample);
+    out << ",\"initialization_seconds\":" << r.initialize_seconds << ",\"mean_staleness\":" << r.mean_staleness
+        << ",\"max_staleness\":" << r.max_staleness << ",\"dataset_load_seconds\":" << r.load_seconds
+        << ",\"training_seconds\":" << r.train_seconds << ",\"sample_seconds\":" << r.sample_seconds
+        << ",\"process_seconds\":" << r.total << ",\"tokens_per_second\":" << tokens / r.train_seconds
+        << ",\"sample_temperature\":1.0,\"d_model\":" << m.d_model << ",\"steps\":" << r.done
+        << ",\"parameters\":" << r.parameters << ",\"final_loss_batches\":" << r.final_loss_batches
+        << ",\"last_loss\":" << r.last_loss << "}";
+}
+
 int run(int argc, char **argv) {
     Options o = parse(argc, argv);
     const TgModelConfig &m = o.model;
@@ -168,11 +265,12 @@ int run(int argc, char **argv) {
     // TRAIN_BYTES_STOP_AFTER=n ends the run after n steps of the same schedule (an interrupted run)
     const char *stop_text = std::getenv("TRAIN_BYTES_STOP_AFTER");
     const int stop = stop_text ? std::min(steps, std::atoi(stop_text)) : steps;
+    const auto process_start = std::chrono::steady_clock::now();
+    std::cout << std::setprecision(9);
     Engine *engine = o.width16 ? tg_create(&m.base) : tg_create_ex(&m);
     if (!engine)
         throw std::runtime_error(tg_error());
     const int64_t count = tg_parameter_count(engine);
-    const auto process_start = std::chrono::steady_clock::now();
 
     std::vector<float> weights, momentum(size_t(count), 0.f), variance(size_t(count), 0.f);
     TgCheckpoint state{};
@@ -204,12 +302,19 @@ int run(int argc, char **argv) {
     check(tg_set_onecycle(engine, &schedule));
     if (state.step > 0)
         check(tg_set_optimizer_state(engine, momentum.data(), variance.data(), state.step));
+    const double initialize_seconds = seconds_since(process_start);
+    // what a resumed run starts from: its rate counts only its own steps and seconds
+    const int start_step = int(state.step);
+    const double start_seconds = state.train_seconds;
 
+    const auto load_start = std::chrono::steady_clock::now();
     std::ifstream file(o.data, std::ios::binary);
     const std::vector<uint8_t> data((std::istreambuf_iterator<char>(file)), std::istreambuf_iterator<char>());
     if (data.empty())
         throw std::runtime_error("cannot read " + o.data);
     check(tg_set_data(engine, data.data(), int64_t(data.size())));
+    const double load_seconds = seconds_since(load_start);
+    log_config(engine, o, schedule, steps, int64_t(data.size()));
 
     TgEventLog *events = nullptr;
     if (!o.log_to.empty()) {
@@ -268,11 +373,11 @@ int run(int argc, char **argv) {
             check(tg_events_scalar(events, "bits-per-byte", tail[m.base.context - 1] / std::log(2.0), at));
             check(tg_events_scalar(events, "lr", double(m.base.learning_rate) * rates.multiplier, at));
             check(tg_events_scalar(events, "mem", used_gb, at));
-            check(tg_events_scalar(events, "tokens_per_second", double(done - int(state.step)) * double(tokens_per_step) /
-                                                                       std::max(train_seconds - state.train_seconds, 1e-9), at));
+            check(tg_events_scalar(events, "tokens_per_second", double(done - start_step) * double(tokens_per_step) /
+                                                                       std::max(train_seconds - start_seconds, 1e-9), at));
         }
-        std::printf("{\"step\": %d, \"loss\": %.6f, \"tokens_per_s\": %.0f}\n", done, last_loss,
-                    double(finished) * double(tokens_per_step) / chunk_seconds);
+        (void)chunk_seconds;
+        log_step(o, schedule, tail, done, train_seconds);
     }
     if (!o.save.empty()) {
         uint64_t optimizer_step = 0;
@@ -284,43 +389,34 @@ int run(int argc, char **argv) {
         state.final_loss_batches = final_batches;
         check(tg_checkpoint_write(o.save.c_str(), &state));
     }
+    const auto sample_start = std::chrono::steady_clock::now();
     const std::string text = done == steps ? sample(engine, m) : "";
+    const double sample_seconds = seconds_since(sample_start);
+    RunReport r{};
+    r.steps = steps, r.done = done, r.final_loss_batches = final_batches, r.sample = text;
+    r.final_losses.resize(size_t(m.base.context));
+    for (int p = 0; p < m.base.context; ++p)
+        r.final_losses[size_t(p)] = final_batches ? final_sums[size_t(p)] / double(final_batches) : double(last_positions[size_t(p)]);
+    r.initialize_seconds = initialize_seconds, r.load_seconds = load_seconds, r.train_seconds = train_seconds;
+    r.sample_seconds = sample_seconds, r.last_loss = last_loss, r.parameters = count;
+    check(tg_pipeline_stats(engine, &r.mean_staleness, &r.max_staleness));
     if (events) {
-        double mean_staleness = 0;
-        int max_staleness = 0;
-        check(tg_pipeline_stats(engine, &mean_staleness, &max_staleness));
         if (!text.empty())
             check(tg_events_text(events, "sample", text.c_str(), int64_t(done) * tokens_per_step));
         check(tg_events_close(events));
-        // report.cpp:83-131; the sample holds printable ASCII without quotes or backslashes
+    }
+    r.total = seconds_since(process_start);
+    std::cout << "{\"summary\":";
+    report(std::cout, o, schedule, r);
+    std::cout << "}" << std::endl;
+    if (events) { // DIR/report.json holds the summary object (report.cpp:119-131)
         const std::string report_path = o.log_to + "/report.json";
-        std::FILE *report = std::fopen(report_path.c_str(), "w");
-        if (!report)
-            throw std::runtime_error("Cannot write " + report_path);
-        const double log2 = std::log(2.0);
-        std::vector<double> average(size_t(m.base.context), 0.0);
-        for (int p = 0; p < m.base.context; ++p)
-            average[size_t(p)] = final_batches ? final_sums[size_t(p)] / double(final_batches) : double(last_positions[size_t(p)]);
-        std::fprintf(report, "{\"architecture\":\"%s\",\"d_model\":%d,\"depth\":%d,\"ctx\":%d,\"batch\":%d,\"inflight\":%d,"
-                             "\"chunk\":%d,\"seed\":%llu,\"optimizer\":\"%s\",\"learning_rate\":%.9g,\"schedule\":\"onecycle\","
-                             "\"schedule_steps\":%d,\"steps\":%d,\"requested_tokens\":%lld,\"tokens\":%lld,\"parameters\":%lld,"
-                             "\"final_loss\":%.9g,\"final_bpb\":%.9g,\"position_bpb\":[",
-                     o.width16 ? "swiglu48-rmsnorm-rope" : "gelu-layernorm-softmax", m.d_model, m.base.depth, m.base.context,
-                     m.base.batch, m.base.inflight, o.chunk, (unsigned long long)m.base.seed, o.width16 ? "muon" : "adamw",
-                     double(m.base.learning_rate), steps, done, o.tokens, 1LL * done * tokens_per_step, (long long)count,
-                     average.back(), average.back() / log2);
-        for (int p = 0; p < m.base.context; ++p)
-            std::fprintf(report, "%s%.9g", p ? "," : "", average[size_t(p)] / log2);
-        std::fprintf(report, "],\"final_loss_batches\":%llu,\"sample\":\"%s\",\"mean_staleness\":%.9g,\"max_staleness\":%d,"
-                             "\"training_seconds\":%.6f,\"process_seconds\":%.6f,\"tokens_per_second\":%.9g}\n",
-                     (unsigned long long)final_batches, text.c_str(), mean_staleness, max_staleness, train_seconds,
-                     seconds_since(process_start),
-                     double(done - int(state.step)) * double(tokens_per_step) / std::max(train_seconds - state.train_seconds, 1e-9));
-        if (std::fclose(report) != 0)
+        std::ofstream out(report_path);
+        report(out, o, schedule, r);
+        out << '\n';
+        if (!out)
             throw std::runtime_error("Cannot write " + report_path);
     }
-    std::printf("{\"steps\": %d, \"final_loss\": %.9g, \"train_seconds\": %.3f, \"sample\": \"%s\"}\n", done, last_loss,
-                train_seconds, text.c_str());
     tg_destroy(engine);
     return 0;
 }
