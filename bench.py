@@ -27,8 +27,20 @@ M = B * T
 # mean over the four projection shapes of 2 * (M*K + N*K + M*N) bytes: operands read and the result written once
 ALGORITHMIC_BYTES_PER_LAUNCH = sum(2 * (M * k + n * k + M * n) for n, k in
                                    [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
-# HBM bytes per launch of that kernel, measured with rocprofv3 FETCH_SIZE / WRITE_SIZE runs of --traffic-probe
-HBM_TRAFFIC_PER_LAUNCH = 151.0e6
+TRAFFIC_PROFILE = "profiles/gemm64_kc_kc_hbm_traffic.md"
+
+
+def hbm_traffic_per_launch():
+    """HBM bytes per launch of the dominant kernel, as the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary of
+    `--traffic-probe` states them ("... = 151.0 MB, against ..."): a figure of that profile, not of this run; None
+    when the file or the line is missing."""
+    import re
+    try:
+        text = open(os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_PROFILE)).read()
+    except OSError:
+        return None
+    found = re.search(r"=\s*([0-9.]+)\s*MB,\s*against", text)
+    return float(found.group(1)) * 1e6 if found else None
 
 
 def gemm_flops():
@@ -312,9 +324,10 @@ def main():
                      "kernel": "gemm64_kernel<128,192,true,true,EpilogueBf16> (forward block projections and "
                                "dgrads: QKV, attention-out, MLP-up, MLP-down)",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": HBM_TRAFFIC_PER_LAUNCH,
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": hbm_traffic_per_launch(),
                      "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE of --traffic-probe, "
                                      "calibrated on a copy of known size)",
+                     "traffic_source": TRAFFIC_PROFILE + " (read from that committed profile, not measured in this run)",
                      "algorithmic_bytes_per_launch": ALGORITHMIC_BYTES_PER_LAUNCH,
                      "flops_per_launch": flops_per_launch, "avg_launch_ms": round(launch_ms, 5)},
         "classes": classes,

@@ -8,8 +8,13 @@
  *     lr_scheduler : total_steps, step, warmup_fraction, initial_lr_fraction, final_lr_fraction,
  *                    low_momentum, high_momentum
  *     trainer      : train_seconds, final_loss_sums, final_loss_batches
- * with the reference's storage numbering (archive/data/0 .. 14, checkpoint.cpp:155-197); the width
- * fields are storages 15 .. 18.  Records are stored uncompressed, 64-byte aligned, with CRC-32.
+ * with the reference's storage numbering (archive/data/0 .. 14, checkpoint.cpp:155-197) and its container
+ * records (.format_version, .storage_alignment, byteorder, version, .data/serialization_id); the width
+ * fields are storages 15 .. 18.  A width-16 file written here loads through the reference's
+ * load_training_state, and a file the reference wrote (storages 0 .. 14 only) reads here as the width-16
+ * network.  Records are stored uncompressed, 64-byte aligned, with CRC-32.  Sizes and offsets are the
+ * 32-bit ZIP fields the reference's reader uses: a file holds less than 4 GiB (about 357 M parameters);
+ * tg_checkpoint_write refuses a larger state before it writes anything.
  * Same status convention as tg_runtime.h: 0 on success, -1 with the reason in tg_error().
  */
 #ifndef TG_CHECKPOINT_H
@@ -42,6 +47,12 @@ TG_API int tg_checkpoint_inspect(const char *path, TgCheckpoint *header);
  * a file whose architecture fields differ from `checkpoint->model` when d_model there is non-zero
  * (checkpoint.cpp:524-551: "Checkpoint architecture mismatch"). */
 TG_API int tg_checkpoint_read(const char *path, TgCheckpoint *checkpoint);
+
+/* The loss summary that travels through checkpoints (FinalLossAverage::add, loss_summary.cpp:5-29): adds the
+ * per-position losses of step `completed_step` (1-based) to sums[positions] and counts it in *batches when the
+ * step lies in the last max(1, ceil(total_steps / 100)) steps of the run; earlier steps change nothing. */
+TG_API int tg_final_loss_add(int total_steps, int positions, int completed_step, const float *losses, double *sums,
+                             uint64_t *batches);
 
 #ifdef __cplusplus
 }

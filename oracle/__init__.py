@@ -13,6 +13,7 @@ import numpy as np
 _HERE = Path(__file__).resolve().parent
 _LIB = None
 _REF = None
+_REF_IO = None
 
 f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
 u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
@@ -58,6 +59,24 @@ def ref_host():
         _REF.tgref_hash_u64.restype = C.c_uint64
         _REF.tgref_hash_u64.argtypes = [C.c_uint64]
     return _REF
+
+
+def ref_io():
+    """The reference's own checkpoint / loss-summary / event-file code behind C linkage (oracle/ref_host_io_shim.cpp),
+    or None when oracle/_ref was never built."""
+    global _REF_IO
+    if _REF_IO is None:
+        path = _HERE / "_ref" / "libtgref_io.so"
+        if not path.exists():
+            return None
+        _REF_IO = C.CDLL(str(path))
+        _REF_IO.tgref_io_error.restype = C.c_char_p
+        _REF_IO.tgref_events_open.restype = C.c_void_p
+        _REF_IO.tgref_events_open.argtypes = [C.c_char_p]
+        _REF_IO.tgref_events_scalar.argtypes = [C.c_void_p, C.c_char_p, C.c_double, C.c_int64]
+        _REF_IO.tgref_events_text.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_int64]
+        _REF_IO.tgref_events_close.argtypes = [C.c_void_p]
+    return _REF_IO
 
 
 def _f(a):

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     engine = declared("tg_runtime.h", "TG_API")
     checkpoint = declared("tg_checkpoint.h", "TG_API")
     events = declared("tg_events.h", "TG_API")
-    assert len(kernel) >= 23 and len(engine) >= 23 and len(checkpoint) == 3 and len(events) == 7
+    assert len(kernel) >= 23 and len(engine) >= 23 and len(checkpoint) == 4 and len(events) == 7
     for name in kernel + engine + checkpoint + events:
         assert hasattr(lib, name), name
     assert set(events) == set(bridge.EVENTS_ABI)

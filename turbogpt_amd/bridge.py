@@ -139,6 +139,7 @@ CHECKPOINT_ABI = {
     "tg_checkpoint_write": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
     "tg_checkpoint_inspect": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
     "tg_checkpoint_read": (i32, [C.c_char_p, C.POINTER(Checkpoint)]),
+    "tg_final_loss_add": (i32, [i32, i32, i32, vp, vp, C.POINTER(u64)]),
 }
 # every symbol include/tg_events.h declares
 EVENTS_ABI = {

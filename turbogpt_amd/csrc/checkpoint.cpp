@@ -151,6 +151,9 @@ Pickle make_pickle(int64_t parameters, int64_t loss_positions) {
 constexpr uint32_t SIG_LOCAL = 0x04034b50, SIG_CENTRAL = 0x02014b50, SIG_END = 0x06054b50,
                    SIG_END64 = 0x06064b50, SIG_LOCATOR64 = 0x07064b50;
 const char *const PREFIX = "archive";
+// the record the reference's reader insists on (checkpoint.cpp:15): 40 characters
+const char *const SERIALIZATION_ID = "3407000000000000000000000000000000000000";
+constexpr uint64_t CHECKPOINT_LIMIT = 0xffffffffull; // sizes and offsets are 32-bit fields
 
 struct FileCloser {
     void operator()(FILE *f) const {
@@ -276,6 +279,7 @@ class ZipReader {
             p += 46 + name_len + extra + comment;
         }
     }
+    bool has(const std::string &name) const { return records_.count(name) != 0; }
     const Record &find(const std::string &name) const {
         const auto it = records_.find(name);
         if (it == records_.end())
@@ -377,8 +381,19 @@ void write_checkpoint(const char *path, const TgCheckpoint &c) {
         {LONG, 1, &s.loss_batches, nullptr}, {LONG, 1, &s.d_model, nullptr},
         {LONG, 1, &s.heads, nullptr},       {LONG, 1, &s.vocab, nullptr},
         {LONG, 1, &s.ffn, nullptr}};
+    // every record and the archive as a whole must fit the 32-bit ZIP fields the reference's reader uses
+    // (checkpoint.cpp:386-411): refuse before anything is written
+    uint64_t total = 1 << 16; // headers, pickle and directory
+    for (int i = 0; i < STORAGES; ++i) {
+        const uint64_t bytes = uint64_t(storages[i].count) * ELEMENT_BYTES[storages[i].kind];
+        if (bytes >= CHECKPOINT_LIMIT)
+            fail("an array of " + std::to_string(bytes) + " bytes does not fit a checkpoint (limit 4 GiB per file)");
+        total += bytes + 256;
+    }
+    if (total >= CHECKPOINT_LIMIT)
+        fail("the model's state (" + std::to_string(total) + " bytes) does not fit a checkpoint (limit 4 GiB per file)");
     const std::string temporary = std::string(path) + ".tmp";
-    {
+    try {
         File file(std::fopen(temporary.c_str(), "wb"));
         if (!file)
             fail("cannot create " + temporary + ": " + std::strerror(errno));
@@ -392,9 +407,13 @@ void write_checkpoint(const char *path, const TgCheckpoint &c) {
         for (int i = 0; i < STORAGES; ++i)
             zip.add(record_name(prefix, i), storages[i].data, uint64_t(storages[i].count) * ELEMENT_BYTES[storages[i].kind]);
         zip.add(prefix + "/version", "3\n");
+        zip.add(prefix + "/.data/serialization_id", SERIALIZATION_ID); // checkpoint.cpp:15,323,519-524
         zip.finish();
         if (std::fflush(file.get()) != 0)
             fail(std::string("write failed: ") + std::strerror(errno));
+    } catch (...) {
+        std::remove(temporary.c_str()); // no partial file stays behind, whatever failed
+        throw;
     }
     if (std::rename(temporary.c_str(), path) != 0) {
         const std::string why = std::strerror(errno);
@@ -414,12 +433,19 @@ std::string read_header(const ZipReader &zip, TgCheckpoint &c) {
         int storage;
         void *out;
     } scalars[] = {{S_DEPTH, &s.depth},       {S_CONTEXT, &s.context},   {S_STEP, &s.step},
-                   {S_TOTAL_STEPS, &s.total_steps}, {S_LOSS_BATCHES, &s.loss_batches}, {S_D_MODEL, &s.d_model},
-                   {S_HEADS, &s.heads},       {S_VOCAB, &s.vocab},       {S_FFN, &s.ffn},
+                   {S_TOTAL_STEPS, &s.total_steps}, {S_LOSS_BATCHES, &s.loss_batches},
                    {S_WARMUP, &s.warmup},     {S_INITIAL, &s.initial},   {S_FINAL, &s.final_fraction},
                    {S_LOW, &s.low},           {S_HIGH, &s.high},         {S_SECONDS, &s.seconds}};
     for (const auto &item : scalars)
         zip.load(record_name(prefix, item.storage), item.out, 8);
+    // The width fields are this library's addition (storages 15 .. 18).  A file the reference wrote has
+    // storages 0 .. 14 only and holds the reference's own network: width 16, 4 heads, vocabulary 256, MLP 48.
+    if (zip.has(record_name(prefix, S_D_MODEL))) {
+        zip.load(record_name(prefix, S_D_MODEL), &s.d_model, 8), zip.load(record_name(prefix, S_HEADS), &s.heads, 8);
+        zip.load(record_name(prefix, S_VOCAB), &s.vocab, 8), zip.load(record_name(prefix, S_FFN), &s.ffn, 8);
+    } else {
+        s.d_model = 16, s.heads = 4, s.vocab = 256, s.ffn = 48;
+    }
     if (s.depth < 1 || s.depth > TG_MAX_DEPTH || s.context < 1 || s.context > (1 << 24) || s.d_model < 1 ||
         s.d_model > (1 << 20) || s.heads < 1 || s.vocab < 1 || s.vocab > (1 << 24) || s.ffn < 1 || s.ffn > (1 << 24) ||
         s.step < 0 || s.total_steps < 0 || s.total_steps > INT32_MAX || s.loss_batches < 0)
@@ -489,5 +515,21 @@ TG_API int tg_checkpoint_read(const char *path, TgCheckpoint *checkpoint) {
         found.weights = checkpoint->weights, found.momentum = checkpoint->momentum;
         found.variance = checkpoint->variance, found.final_loss_sums = checkpoint->final_loss_sums;
         *checkpoint = found;
+    });
+}
+
+// The loss summary a run carries through its checkpoints (loss_summary.cpp:5-29): per-position sums over the
+// steps after total_steps - max(1, ceil(total_steps / 100)).
+TG_API int tg_final_loss_add(int total_steps, int positions, int completed_step, const float *losses, double *sums,
+                             uint64_t *batches) {
+    return guarded([&] {
+        require(total_steps >= 0 && positions > 0 && losses && sums && batches, "final loss: missing argument");
+        const int window = (total_steps + 99) / 100 > 1 ? (total_steps + 99) / 100 : 1;
+        const int first_step = total_steps > window ? total_steps - window : 0;
+        if (completed_step <= first_step)
+            return;
+        for (int p = 0; p < positions; ++p)
+            sums[p] += losses[p];
+        ++*batches;
     });
 }

@@ -278,7 +278,6 @@ int run(int argc, char **argv) {
     OneCycle schedule{steps, 0.3, 0.04, 0.000004, 0.85, 0.95};
     // loss averaged over the last max(1, ceil(steps / 100)) steps, carried through checkpoints
     // (loss_summary.cpp:5-29)
-    const int average_after = std::max(0, steps - std::max(1, (steps + 99) / 100));
     std::vector<double> final_sums(size_t(m.base.context), 0.0);
     uint64_t final_batches = 0;
     if (o.load.empty()) {
@@ -355,13 +354,9 @@ int run(int argc, char **argv) {
         const float *tail = history.data() + size_t(finished - 1) * size_t(m.base.context);
         last_loss = std::accumulate(tail, tail + m.base.context, 0.0) / m.base.context;
         std::copy(tail, tail + m.base.context, last_positions.begin());
-        for (int i = 0; i < finished; ++i) {
-            if (done - finished + i + 1 <= average_after)
-                continue;
-            for (int p = 0; p < m.base.context; ++p)
-                final_sums[size_t(p)] += history[size_t(i) * size_t(m.base.context) + size_t(p)];
-            ++final_batches;
-        }
+        for (int i = 0; i < finished; ++i)
+            check(tg_final_loss_add(steps, m.base.context, done - finished + i + 1,
+                                    history.data() + size_t(i) * size_t(m.base.context), final_sums.data(), &final_batches));
         if (events) { // training_log.cpp:75-97; the step axis counts tokens
             const int64_t at = int64_t(done) * tokens_per_step;
             StepRates rates{};
