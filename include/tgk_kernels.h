@@ -160,6 +160,17 @@ TGK_API int tgk_layernorm_bwd_add(hipStream_t stream, int rows, int D, const uin
                                   uint16_t *dx, float *dgamma, float *dbeta, float eps, int accumulate,
                                   void *workspace, size_t workspace_bytes);
 TGK_API size_t tgk_layernorm_bwd_workspace(int rows, int D);
+/* The two halves of tgk_layernorm_bwd_add, for a caller that runs many LayerNorm backwards before it needs
+ * their parameter gradients (a training step has 2 * depth + 1): _rows writes dx and this LayerNorm's partial
+ * sums (tgk_layernorm_bwd_workspace(rows, D) bytes at `partials`, which must stay untouched until the fold);
+ * _fold sums `count` such partial blocks, job j at partials + j * job_stride_bytes, into the dgamma / dbeta
+ * pointer pairs of a DEVICE array `targets` ({float *dgamma, *dbeta} per job) in one launch.  Same sums in the
+ * same order as tgk_layernorm_bwd_add: the gradients are bit-identical. */
+TGK_API int tgk_layernorm_bwd_rows(hipStream_t stream, int rows, int D, const uint16_t *x, const uint16_t *dy,
+                                   const uint16_t *gamma_hi, const uint16_t *gamma_lo, const uint16_t *residual,
+                                   uint16_t *dx, float eps, void *partials, size_t partials_bytes);
+TGK_API int tgk_layernorm_bwd_fold(hipStream_t stream, int rows, int D, int count, const void *partials,
+                                   size_t job_stride_bytes, const void *targets, int accumulate);
 
 /* Softmax cross-entropy over 256 byte classes on bf16 logits [rows][256] (cuda/model.cuh:33-58):
  * loss[t] = logsumexp - logit[y[t]]; logits_f32 (optional) receives the logits as fp32;

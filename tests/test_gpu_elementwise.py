@@ -95,6 +95,46 @@ def test_layernorm_forward_backward(orc, M, D):
         assert np.array_equal(host(prior), ph)
 
 
+def test_layernorm_backward_in_two_halves_equals_the_single_call(orc):
+    """tgk_layernorm_bwd_rows for three LayerNorms, then ONE tgk_layernorm_bwd_fold: dx and the parameter gradients
+    equal three tgk_layernorm_bwd_add calls bit for bit (same partial sums, same order of additions)."""
+    lib = library()
+    M, D, jobs = 333, 768, 3
+    rng = np.random.default_rng(12)
+    stride = lib.tgk_layernorm_bwd_workspace(M, D)
+    partials = torch.empty(jobs * stride, dtype=torch.uint8, device="cuda")
+    ws = torch.empty(stride, dtype=torch.uint8, device="cuda")
+    got = torch.full((jobs, 2, D), 7.0, dtype=torch.float32, device="cuda")
+    want = torch.full((jobs, 2, D), 7.0, dtype=torch.float32, device="cuda")
+    table = torch.tensor([[got[j, 0].data_ptr(), got[j, 1].data_ptr()] for j in range(jobs)], dtype=torch.int64,
+                         device="cuda")
+    keep = []
+    for j in range(jobs):
+        x, _ = to_bf16_device(rng.standard_normal((M, D)) * (1 + j))
+        dy, _ = to_bf16_device(rng.standard_normal((M, D)))
+        residual, _ = to_bf16_device(rng.standard_normal((M, D)))
+        gh, gl = hilo(orc, (1 + 0.2 * rng.standard_normal(D)).astype(np.float32))
+        dx_a, dx_b = torch.empty_like(x), torch.empty_like(x)
+        with_residual = residual.data_ptr() if j != 1 else None
+        check(lib.tgk_layernorm_bwd_rows(stream(), M, D, x.data_ptr(), dy.data_ptr(), gh.data_ptr(), gl.data_ptr(),
+                                         with_residual, dx_a.data_ptr(), 1e-5, partials.data_ptr() + j * stride, stride))
+        check(lib.tgk_layernorm_bwd_add(stream(), M, D, x.data_ptr(), dy.data_ptr(), gh.data_ptr(), gl.data_ptr(),
+                                        with_residual, dx_b.data_ptr(), want[j, 0].data_ptr(), want[j, 1].data_ptr(), 1e-5, 0,
+                                        ws.data_ptr(), stride))
+        keep.append((x, dy, residual, gh, gl, dx_a, dx_b))
+    check(lib.tgk_layernorm_bwd_fold(stream(), M, D, jobs, partials.data_ptr(), stride, table.data_ptr(), 0))
+    sync()
+    for _, _, _, _, _, dx_a, dx_b in keep:
+        assert torch.equal(dx_a, dx_b)
+    assert torch.equal(got, want) and float(got.abs().sum()) > 0 and not bool((got == 7.0).any())
+    # accumulate adds to what is there
+    check(lib.tgk_layernorm_bwd_fold(stream(), M, D, jobs, partials.data_ptr(), stride, table.data_ptr(), 1))
+    sync()
+    assert torch.equal(got, want + want)
+    # a job stride below one LayerNorm's partial block is refused on the host
+    assert lib.tgk_layernorm_bwd_fold(stream(), M, D, jobs, partials.data_ptr(), stride - 16, table.data_ptr(), 0) == -1
+
+
 def test_cross_entropy_loss_logits_and_gradient(orc):
     lib = library()
     rng = np.random.default_rng(17)

@@ -39,6 +39,8 @@ KERNEL_ABI = {
     "tgk_layernorm_bwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, f32, i32, i32, vp, sz]),
     "tgk_layernorm_bwd_add": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, f32, i32, vp, sz]),
     "tgk_layernorm_bwd_workspace": (sz, [i32, i32]),
+    "tgk_layernorm_bwd_rows": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, f32, vp, sz]),
+    "tgk_layernorm_bwd_fold": (i32, [vp, i32, i32, i32, vp, sz, vp, i32]),
     "tgk_cross_entropy": (i32, [vp, i32, i32, vp, vp, vp, vp, f32, i32]),
     "tgk_sumsq_partials": (i32, [vp, vp, sz, vp, i32]),
     "tgk_adamw": (i32, [vp, sz, vp, vp, vp, vp, vp, vp, i32, vp, vp, i32, f32, f32, f32, f32, f32, f32,

@@ -385,6 +385,45 @@ __global__ __launch_bounds__(256) void layernorm_bwd_reduce_kernel(const float *
     }
 }
 
+// The same fold for many LayerNorms in one launch: job j sums the partial rows at partial + j * job_stride into
+// its own dgamma / dbeta (device array of pointer pairs).  blockIdx.y selects the job.  Same order of additions
+// as layernorm_bwd_reduce_kernel, so a gradient folded here equals one folded there bit for bit.
+struct LayerNormFoldTarget {
+    float *dgamma, *dbeta;
+};
+__global__ __launch_bounds__(256) void layernorm_bwd_fold_batch_kernel(const float *__restrict__ partial,
+                                                                       size_t job_stride, int blocks, int D,
+                                                                       const LayerNormFoldTarget *__restrict__ targets,
+                                                                       int accumulate) {
+    __shared__ float part[16][17];
+    const float *mine = partial + size_t(blockIdx.y) * job_stride;
+    const int col = threadIdx.x & 15, phase = threadIdx.x >> 4, i = blockIdx.x * 16 + col;
+    const size_t row_stride = size_t(2) * D;
+    float s[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        s[u] = 0.f;
+    int b = phase;
+    for (; b + 16 * 7 < blocks; b += 16 * 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            s[u] += mine[size_t(b + 16 * u) * row_stride + i];
+    }
+    for (; b < blocks; b += 16)
+        s[0] += mine[size_t(b) * row_stride + i];
+    part[phase][col] = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
+    __syncthreads();
+    if (phase == 0) {
+        float sum = 0.f;
+#pragma unroll
+        for (int p = 0; p < 16; ++p)
+            sum += part[p][col];
+        const LayerNormFoldTarget t = targets[blockIdx.y];
+        float *out = i < D ? t.dgamma + i : t.dbeta + (i - D);
+        *out = accumulate ? *out + sum : sum;
+    }
+}
+
 // ---- cross-entropy over 256 byte classes ------------------------------------------------------
 // One wave per token: loss, optional fp32 copy of the logits, dlogits = RN((softmax - onehot) * k)
 // written in place over the bf16 logits (cuda/model.cuh:33-58).
@@ -723,42 +762,76 @@ static int layernorm_bwd_blocks(int rows) {
 extern "C" size_t tgk_layernorm_bwd_workspace(int rows, int D) {
     return rows > 0 && D > 0 ? size_t(layernorm_bwd_blocks(rows)) * 2 * D * sizeof(float) : 0;
 }
+namespace {
+// the row kernel: dx, and one partial row pair (dgamma | dbeta) per block into `partial`
+void launch_layernorm_bwd_rows(hipStream_t stream, int rows, int D, const uint16_t *x, const uint16_t *dy,
+                               const uint16_t *gamma_hi, const uint16_t *gamma_lo, const uint16_t *residual, uint16_t *dx,
+                               float eps, float *partial) {
+    require(rows > 0 && D > 0 && D % 64 == 0 && D <= MAX_LN_CHUNKS * 512,
+            "layernorm_bwd: D must be a multiple of 64, at most 2048");
+    aligned(x, "layernorm: x");
+    aligned(dy, "layernorm: dy");
+    aligned(dx, "layernorm: dx");
+    aligned(gamma_hi, "layernorm: gamma_hi");
+    aligned(gamma_lo, "layernorm: gamma_lo");
+    if (residual)
+        aligned(residual, "layernorm: residual");
+    const int blocks = layernorm_bwd_blocks(rows);
+    // one row per wave here: two rows per wave cost registers (148 for D = 768) and LDS that lower the
+    // occupancy, and measured slower
+    const int per_lane = (D / 8 + 63) / 64;
+    const size_t lds = size_t(4) * 2 * D * sizeof(float);
+#define TG_LN_BWD(NC, GROUP)                                                                                      \
+    hipLaunchKernelGGL((layernorm_bwd_kernel<NC, GROUP>), dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,  \
+                       gamma_lo, residual, dx, partial, rows, D, eps)
+    if (per_lane == 1)
+        TG_LN_BWD(1, 64);
+    else if (per_lane == 2)
+        TG_LN_BWD(2, 64);
+    else
+        TG_LN_BWD(4, 64);
+#undef TG_LN_BWD
+    check_hip(hipGetLastError(), "layernorm_bwd launch: ");
+}
+} // namespace
+
 extern "C" int tgk_layernorm_bwd_add(hipStream_t stream, int rows, int D, const uint16_t *x,
                                      const uint16_t *dy, const uint16_t *gamma_hi, const uint16_t *gamma_lo,
                                      const uint16_t *residual, uint16_t *dx, float *dgamma, float *dbeta,
                                      float eps, int accumulate, void *workspace, size_t workspace_bytes) {
     return guarded([&] {
-        require(rows > 0 && D > 0 && D % 64 == 0 && D <= MAX_LN_CHUNKS * 512,
-                "layernorm_bwd: D must be a multiple of 64, at most 2048");
-        aligned(x, "layernorm: x");
-        aligned(dy, "layernorm: dy");
-        aligned(dx, "layernorm: dx");
-        aligned(gamma_hi, "layernorm: gamma_hi");
-        aligned(gamma_lo, "layernorm: gamma_lo");
-        if (residual)
-            aligned(residual, "layernorm: residual");
         require(dgamma && dbeta, "layernorm_bwd: missing operand");
         require(workspace && workspace_bytes >= tgk_layernorm_bwd_workspace(rows, D),
                 "layernorm_bwd: workspace too small (see tgk_layernorm_bwd_workspace)");
-        const int blocks = layernorm_bwd_blocks(rows);
         float *partial = static_cast<float *>(workspace);
-        // one row per wave here: two rows per wave cost registers (148 for D = 768) and LDS that lower the
-        // occupancy, and measured slower
-        const int per_lane = (D / 8 + 63) / 64;
-        const size_t lds = size_t(4) * 2 * D * sizeof(float);
-#define TG_LN_BWD(NC, GROUP)                                                                                      \
-    hipLaunchKernelGGL((layernorm_bwd_kernel<NC, GROUP>), dim3(blocks), dim3(256), lds, stream, x, dy, gamma_hi,  \
-                       gamma_lo, residual, dx, partial, rows, D, eps)
-        if (per_lane == 1)
-            TG_LN_BWD(1, 64);
-        else if (per_lane == 2)
-            TG_LN_BWD(2, 64);
-        else
-            TG_LN_BWD(4, 64);
-#undef TG_LN_BWD
-        hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3(2 * D / 16), dim3(256), 0, stream, partial, blocks, D,
-                           dgamma, dbeta, accumulate);
+        launch_layernorm_bwd_rows(stream, rows, D, x, dy, gamma_hi, gamma_lo, residual, dx, eps, partial);
+        hipLaunchKernelGGL(layernorm_bwd_reduce_kernel, dim3(2 * D / 16), dim3(256), 0, stream, partial,
+                           layernorm_bwd_blocks(rows), D, dgamma, dbeta, accumulate);
         check_hip(hipGetLastError(), "layernorm_bwd launch: ");
+    });
+}
+extern "C" int tgk_layernorm_bwd_rows(hipStream_t stream, int rows, int D, const uint16_t *x, const uint16_t *dy,
+                                      const uint16_t *gamma_hi, const uint16_t *gamma_lo, const uint16_t *residual,
+                                      uint16_t *dx, float eps, void *partials, size_t partials_bytes) {
+    return guarded([&] {
+        require(partials && partials_bytes >= tgk_layernorm_bwd_workspace(rows, D) &&
+                    !(reinterpret_cast<uintptr_t>(partials) & 15),
+                "layernorm_bwd_rows: partials too small (see tgk_layernorm_bwd_workspace)");
+        launch_layernorm_bwd_rows(stream, rows, D, x, dy, gamma_hi, gamma_lo, residual, dx, eps,
+                                  static_cast<float *>(partials));
+    });
+}
+extern "C" int tgk_layernorm_bwd_fold(hipStream_t stream, int rows, int D, int count, const void *partials,
+                                      size_t job_stride_bytes, const void *targets, int accumulate) {
+    return guarded([&] {
+        require(rows > 0 && D > 0 && D % 64 == 0 && count > 0 && count <= 65535, "layernorm_bwd_fold: bad shape");
+        require(partials && targets && job_stride_bytes % 16 == 0 &&
+                    job_stride_bytes >= tgk_layernorm_bwd_workspace(rows, D),
+                "layernorm_bwd_fold: missing operand or job stride below tgk_layernorm_bwd_workspace");
+        hipLaunchKernelGGL(layernorm_bwd_fold_batch_kernel, dim3(2 * D / 16, count), dim3(256), 0, stream,
+                           static_cast<const float *>(partials), job_stride_bytes / sizeof(float),
+                           layernorm_bwd_blocks(rows), D, static_cast<const LayerNormFoldTarget *>(targets), accumulate);
+        check_hip(hipGetLastError(), "layernorm_bwd_fold launch: ");
     });
 }
 extern "C" int tgk_layernorm_bwd(hipStream_t stream, int rows, int D, const uint16_t *x,

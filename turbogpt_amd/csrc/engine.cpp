@@ -71,6 +71,10 @@ struct Slot {
     bf16_t *nf = nullptr, *logits = nullptr, *dh = nullptr, *t1 = nullptr, *du = nullptr, *dqkv = nullptr;
     bf16_t *dh_mid = nullptr; // the gradient between a block's two halves, when the block's weight gradients are batched
     void *workspace = nullptr;
+    // LayerNorm parameter gradients: every LayerNorm backward of a step leaves its per-block partial sums in a
+    // block of its own here and one launch at the end of the backward pass folds all 2 * depth + 1 of them
+    uint8_t *ln_partials = nullptr;
+    void *ln_targets = nullptr; // device array of {dgamma, dbeta} pointers into `gradient`, in fold order
 };
 // One immutable copy of the weights: a batch reads a single version from its first kernel to its last
 // (cuda/pipeline.cuh:36-38).  inflight = K keeps K + 1 of them in a ring; a synchronous engine one.
@@ -272,8 +276,14 @@ struct Engine {
         float *g = gradient;
         OP(TG_CLASS_HEAD, tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
         OP(TG_CLASS_HEAD, tgk_gemm_dgrad_t(stream, M, V, d, logits, V, wt(layout.head), V, t1, d, nullptr, 0));
-        OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, x[c.depth], t1, w(layout.lnf_g), wl(layout.lnf_g), dh,
-                             g + layout.lnf_g, g + layout.lnf_b, config.ln_eps, 0, 0, workspace, workspace_bytes));
+        // LayerNorm j of the fold: 0 = final, 1 + 2 l = block l's second, 2 + 2 l = its first
+        const size_t ln_stride = tgk_layernorm_bwd_workspace(M, d);
+        const auto ln_rows = [&](int job, const bf16_t *input, const bf16_t *dy, int64_t gamma, const bf16_t *residual,
+                                 bf16_t *dx) {
+            return tgk_layernorm_bwd_rows(stream, M, d, input, dy, w(gamma), wl(gamma), residual, dx, config.ln_eps,
+                                          s.ln_partials + size_t(job) * ln_stride, ln_stride);
+        };
+        OP(TG_CLASS_LAYERNORM_BWD, ln_rows(0, x[c.depth], t1, layout.lnf_g, nullptr, dh));
         for (int l = c.depth - 1; l >= 0; --l) {
             const TgLayerParameters &p = layout.layers[l];
             LayerBuffers &b = layers[l];
@@ -284,9 +294,7 @@ struct Engine {
                 bf16_t *mid = s.dh_mid;
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, du, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
-                OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_add(stream, M, d, b.mid, t1, w(p.ln2_g), wl(p.ln2_g), dh, mid,
-                                                                 g + p.ln2_g, g + p.ln2_b, config.ln_eps, 0, workspace,
-                                                                 workspace_bytes));
+                OP(TG_CLASS_LAYERNORM_BWD, ln_rows(1 + 2 * l, b.mid, t1, p.ln2_g, dh, mid));
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, d, mid, d, wt(p.attn_out), d, t1, d, nullptr, 0));
                 OP(TG_CLASS_ATTN_BWD, tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d,
                                                    b.qkv + 2 * d, 3 * d, b.o, d, b.lse, t1, d, dqkv, dqkv + d, dqkv + 2 * d,
@@ -297,17 +305,14 @@ struct Engine {
                                              {3 * d, d, dqkv, 3 * d, b.n1, d, g + p.qkv, d}};
                 OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad_batch(stream, M, 4, jobs, 0, workspace, workspace_bytes));
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, 3 * d, d, dqkv, 3 * d, wt(p.qkv), 3 * d, t1, d, nullptr, 0));
-                OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_add(stream, M, d, x[l], t1, w(p.ln1_g), wl(p.ln1_g), mid, dh,
-                                                                 g + p.ln1_g, g + p.ln1_b, config.ln_eps, 0, workspace,
-                                                                 workspace_bytes));
+                OP(TG_CLASS_LAYERNORM_BWD, ln_rows(2 + 2 * l, x[l], t1, p.ln1_g, mid, dh));
                 continue;
             }
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, F, dh, d, b.a, F, g + p.mlp_down, F, 0, workspace, workspace_bytes));
             OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, F, d, du, F, b.n2, d, g + p.mlp_up, d, 0, workspace, workspace_bytes));
             OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, du, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
-            OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, b.mid, t1, w(p.ln2_g), wl(p.ln2_g), dh, g + p.ln2_g, g + p.ln2_b,
-                                 config.ln_eps, 1, 0, workspace, workspace_bytes));
+            OP(TG_CLASS_LAYERNORM_BWD, ln_rows(1 + 2 * l, b.mid, t1, p.ln2_g, dh, dh));
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, d, dh, d, b.o, d, g + p.attn_out, d, 0, workspace, workspace_bytes));
             OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, d, dh, d, wt(p.attn_out), d, t1, d, nullptr, 0));
             OP(TG_CLASS_ATTN_BWD, tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d, b.qkv + 2 * d,
@@ -316,9 +321,9 @@ struct Engine {
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, 3 * d, d, dqkv, 3 * d, b.n1, d, g + p.qkv, d, 0, workspace,
                               workspace_bytes));
             OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, 3 * d, d, dqkv, 3 * d, wt(p.qkv), 3 * d, t1, d, nullptr, 0));
-            OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd(stream, M, d, x[l], t1, w(p.ln1_g), wl(p.ln1_g), dh, g + p.ln1_g, g + p.ln1_b,
-                                 config.ln_eps, 1, 0, workspace, workspace_bytes));
+            OP(TG_CLASS_LAYERNORM_BWD, ln_rows(2 + 2 * l, x[l], t1, p.ln1_g, dh, dh));
         }
+        OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_fold(stream, M, d, 2 * c.depth + 1, s.ln_partials, ln_stride, s.ln_targets, 0));
         OP(TG_CLASS_OTHER, tgk_embed_bwd(stream, c.batch, T, d, V, tokens_in, dh, g + layout.embedding, g + layout.positions, 0,
                                          workspace, workspace_bytes));
     }
@@ -672,10 +677,24 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(d), int(d)));
         need = std::max(need, tgk_gemm_wgrad_workspace(int(M), int(3 * d), int(d)));
         e->workspace_bytes = need;
+        const int norms = 2 * c.depth + 1;
+        const size_t ln_stride = tgk_layernorm_bwd_workspace(int(M), int(d));
         for (Slot &slot : e->slots) {
             uint8_t *ws = nullptr;
             e->allocate(ws, need, false);
             slot.workspace = ws;
+            e->allocate(slot.ln_partials, size_t(norms) * ln_stride, false);
+            std::vector<float *> targets(size_t(2 * norms));
+            targets[0] = slot.gradient + e->layout.lnf_g, targets[1] = slot.gradient + e->layout.lnf_b;
+            for (int l = 0; l < c.depth; ++l) {
+                const TgLayerParameters &p = e->layout.layers[l];
+                targets[size_t(2 * (1 + 2 * l))] = slot.gradient + p.ln2_g, targets[size_t(2 * (1 + 2 * l) + 1)] = slot.gradient + p.ln2_b;
+                targets[size_t(2 * (2 + 2 * l))] = slot.gradient + p.ln1_g, targets[size_t(2 * (2 + 2 * l) + 1)] = slot.gradient + p.ln1_b;
+            }
+            uint8_t *table = nullptr;
+            e->allocate(table, targets.size() * sizeof(float *), false);
+            check_hip(hipMemcpy(table, targets.data(), targets.size() * sizeof(float *), hipMemcpyHostToDevice));
+            slot.ln_targets = table;
         }
         e->sync();
         return e;
