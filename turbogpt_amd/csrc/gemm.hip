@@ -15,9 +15,10 @@
 // list of work items (tile x split).  LDS tiles are unpadded and XOR-swizzled on 16-byte chunks (a wave-wide
 // copy fills 1 KiB of LDS contiguously, so padding is not available); measured bank conflicts are zero.
 // k-contiguous tiles give each MFMA fragment with one ds_read_b128; k-strided tiles keep the natural [k][row]
-// image and are read with the transposing ds_read_b64_tr_b16.  256 threads = 2x2 waves of
-// v_mfma_f32_32x32x16_bf16; the instruction's A operand is fed with *our B rows* so that a lane ends up holding
-// 4 consecutive n for one m.  Results leave through a wave-private LDS transposition so that stores cover
+// image and are read with the transposing ds_read_b64_tr_b16.  256 threads = 2x2 waves; the 64-k kernels use
+// v_mfma_f32_16x16x32_bf16 (more flops per watt on real operands, and the kernels run against the power limit),
+// gemm_kernel v_mfma_f32_32x32x16_bf16; either way the instruction's A operand is fed with *our B rows* so that a
+// lane ends up holding 4 consecutive n for one m.  Results leave through a wave-private LDS transposition so that stores cover
 // whole row pieces, with the residual / GELU / GELU' epilogues applied in that layout.
 //
 // Three kernels: gemm64_kernel (two stages of 64 k, copies placed between the MFMAs: every training shape),
@@ -169,6 +170,69 @@ TG_DEVICE void staged_store_f32(const f32x16 (&acc)[FM][FN], unsigned char *mine
         }
 }
 
+// The same two stores for accumulators kept as 2 x 2 tiles of 16 x 16 per 32 x 32 block (v_mfma_f32_16x16x32_bf16 fed
+// with B rows as its first operand): tile [tm][tn] of a block holds, in lane l, row m = 16 tm + l % 16 and columns
+// n = 16 tn + 4 (l / 16) .. + 3.
+template <int FM, int FN, class Epilogue>
+TG_DEVICE void staged_store_bf16(const f32x4 (&acc)[FM][FN][2][2], const u32x4 (&first)[2], unsigned char *mine,
+                                 const Epilogue &epilogue, int m_base, int n_base, int lane) {
+    const int get_row = lane >> 2, get_chunk = lane & 3;
+    const int row = lane & 15;
+    unsigned char *put = mine + row * 64 + ((lane >> 4) & 1) * 8;
+    const int put_swizzle = (row >> 2) & 3, put_chunk = lane >> 5;
+    const unsigned char *get = mine + get_row * 64 + ((get_chunk ^ ((get_row >> 2) & 3)) << 4);
+    const bool wants_aux = epilogue.wants_aux();
+    u32x4 aux[2] = {first[0], first[1]};
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            u32x4 next[2] = {aux[0], aux[1]};
+            if (wants_aux && i * FN + j + 1 < FM * FN)
+                load_aux_pair<FM, FN>(epilogue, i * FN + j + 1, m_base, n_base, lane, next);
+            const int m = m_base + i * 32 + get_row, n = n_base + j * 32 + get_chunk * 8;
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < 2; ++tn) {
+                    const f32x4 &t = acc[i][j][tm][tn];
+                    u32x2 packed;
+                    packed.x = pack_bf16(t[0], t[1]);
+                    packed.y = pack_bf16(t[2], t[3]);
+                    *reinterpret_cast<u32x2 *>(put + tm * 1024 + (((2 * tn + put_chunk) ^ put_swizzle) << 4)) = packed;
+                }
+            epilogue.finish(m, n, *reinterpret_cast<const u32x4 *>(get), aux[0]);
+            epilogue.finish(m + 16, n, *reinterpret_cast<const u32x4 *>(get + 1024), aux[1]);
+            aux[0] = next[0];
+            aux[1] = next[1];
+        }
+}
+template <int FM, int FN, class Epilogue>
+TG_DEVICE void staged_store_f32(const f32x4 (&acc)[FM][FN][2][2], unsigned char *mine, const Epilogue &epilogue,
+                                int m_base, int n_base, int lane, int split) {
+    const int row = lane & 15;
+    unsigned char *put = mine + row * 128;
+    const int put_swizzle = (row >> 1) & 7, put_chunk = lane >> 4;
+    const int first_row = lane >> 3, chunk = lane & 7;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+#pragma unroll
+            for (int tm = 0; tm < 2; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < 2; ++tn)
+                    *reinterpret_cast<f32x4 *>(put + tm * 2048 + (((4 * tn + put_chunk) ^ put_swizzle) << 4)) =
+                        acc[i][j][tm][tn];
+#pragma unroll
+            for (int part = 0; part < 4; ++part) {
+                const int r = first_row + part * 8;
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(mine + r * 128 + ((chunk ^ ((r >> 1) & 7)) << 4));
+                epilogue.finish(m_base + i * 32 + r, n_base + j * 32 + chunk * 4, v, split);
+            }
+        }
+}
+
 constexpr int BK = 32;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -203,8 +267,9 @@ template <int ROWS> struct TileKS {
     static constexpr int BYTES = ROWS * 64;
     static constexpr int CHUNKS_PER_ROW = ROWS / 8;
     TG_DEVICE static int swizzle(int r) {
-        // row stride of 256 B multiples: 4 consecutive k-rows start in the same bank; 384 B: every other one
-        return ROWS % 128 == 0 ? ((r & 3) << 2) : (((r >> 1) & 1) << 2);
+        // row stride of 256 B multiples: 4 consecutive k-rows start in the same bank; 384 B: every other one.  The
+        // 16-row fragments read k-rows r and r + 8 in one pass, 32 bytes of each: bit 3 of r moves them 32 bytes apart.
+        return (ROWS % 128 == 0 ? ((r & 3) << 2) : (((r >> 1) & 1) << 2)) | (((r >> 3) & 1) << 1);
     }
     TG_DEVICE static int64_t source_offset(int j, int tid, int ld) {
         const int wave = tid >> 6, lane = tid & 63;
@@ -224,6 +289,18 @@ template <int ROWS> struct TileKS {
         const unsigned char *p = tile + r * (ROWS * 2) + chunk * 16 + (i & 1) * 8;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * ROWS * 2));
+        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, both);
+    }
+    // fragment of a 16-column tile: columns row0 + lane%16, k = k0 + 8*(lane/16) .. +7
+    TG_DEVICE static bf16x8 frag16(const unsigned char *tile, int row0, int k0, int lane) {
+        const int g = lane >> 4, i = lane & 15;
+        const int r = k0 + 8 * g + (i >> 2);
+        const int col = row0 + 4 * (i & 3);
+        const unsigned char *p = tile + r * (ROWS * 2) + (i & 1) * 8;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + (((col >> 3) ^ swizzle(r)) << 4)));
+        const s16x4 hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * ROWS * 2 + (((col >> 3) ^ swizzle(r + 4)) << 4)));
         const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         return __builtin_bit_cast(bf16x8, both);
     }
@@ -433,6 +510,11 @@ template <int ROWS> struct TileKC64 {
         const int row = row0 + (lane & 31), chunk = (ks * 2 + (lane >> 5)) ^ ((row >> 1) & 7);
         return *reinterpret_cast<const bf16x8 *>(tile + row * 128 + chunk * 16);
     }
+    // fragment of a 16-row tile for the 32-k step ks (0..1): rows row0 + lane%16, k = ks*32 + 8*(lane/16) .. +7
+    TG_DEVICE static bf16x8 frag16(const unsigned char *tile, int row0, int ks, int lane) {
+        const int row = row0 + (lane & 15), chunk = (ks * 4 + (lane >> 4)) ^ ((row >> 1) & 7);
+        return *reinterpret_cast<const bf16x8 *>(tile + row * 128 + chunk * 16);
+    }
 };
 // k-strided tile: 64 k-rows x ROWS columns in the natural [k][row] image, swizzled and read like TileKS
 template <int ROWS> struct TileKS64 {
@@ -451,47 +533,50 @@ template <int ROWS> struct TileKS64 {
     TG_DEVICE static bf16x8 frag(const unsigned char *tile, int row0, int ks, int lane) {
         return TileKS<ROWS>::frag(tile, row0, ks, lane); // k-rows ks*16 .. of the 64
     }
+    TG_DEVICE static bf16x8 frag16(const unsigned char *tile, int row0, int ks, int lane) {
+        return TileKS<ROWS>::frag16(tile, row0, ks * 32, lane); // k-rows ks*32 .. of the 64
+    }
 };
 template <int ROWS, bool KC> struct Tile64Of;
 template <int ROWS> struct Tile64Of<ROWS, true> { using type = TileKC64<ROWS>; };
 template <int ROWS> struct Tile64Of<ROWS, false> { using type = TileKS64<ROWS>; };
 
-// One 64-k stage of a wave's FM x FN tiles: fragments of the next 16-k step are read while the current MFMAs
-// run, and copy number n of the next stage goes out behind MFMA n (see gemm64_kernel).
+// One 64-k stage of a wave's FM x FN blocks of 32 x 32 with v_mfma_f32_16x16x32_bf16: two 32-k steps, every block as
+// 2 x 2 tiles of 16 x 16.  The kernels run against the board's power limit, and on random operands this instruction
+// sustains about 15 % more than the 32x32x16 form at the same power (measured from registers: 2.06 against 1.79
+// PFLOP/s; it moves half the accumulator bytes per flop).  Copy n of the next stage goes out behind matrix
+// instruction 2n (see gemm64_kernel).
 template <class TA, class TB, int FM, int FN, int LOADS, class Copy>
-TG_DEVICE void multiply_stage(f32x16 (&acc)[FM][FN], const unsigned char *slot, int wm, int wn, int lane, bool copy,
-                              Copy &&copy_one) {
+TG_DEVICE void multiply_stage(f32x4 (&acc)[FM][FN][2][2], const unsigned char *slot, int wm, int wn, int lane,
+                                bool copy, Copy &&copy_one) {
+    // A column = one 16-row B fragment against the 2 FM A fragments of its 32-k step.  The A fragments of both steps
+    // are held (the second step's are read during the first), B fragments are read one column ahead.
+    constexpr int AF = 2 * FM, BF = 2 * FN, COLUMNS = 2 * BF;
     const unsigned char *sa = slot, *sb = sa + TA::BYTES;
-    bf16x8 af[2][FM], bfr[2][FN];
+    bf16x8 af[2][AF], bfr[2];
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
-        af[0][i] = TA::frag(sa, wm + i * 32, 0, lane);
+    for (int i = 0; i < AF; ++i)
+        af[0][i] = TA::frag16(sa, wm + i * 16, 0, lane);
+    bfr[0] = TB::frag16(sb, wn, 0, lane);
 #pragma unroll
-    for (int j = 0; j < FN; ++j)
-        bfr[0][j] = TB::frag(sb, wn + j * 32, 0, lane);
+    for (int column = 0; column < COLUMNS; ++column) {
+        const int ks = column / BF, j = column % BF;
+        if (column + 1 < COLUMNS)
+            bfr[(column + 1) & 1] = TB::frag16(sb, wn + ((column + 1) % BF) * 16, (column + 1) / BF, lane);
+        if (ks == 0 && j < AF)
+            af[1][j] = TA::frag16(sa, wm + j * 16, 1, lane);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        if (ks < 3) {
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-                af[(ks + 1) & 1][i] = TA::frag(sa, wm + i * 32, ks + 1, lane);
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-                bfr[(ks + 1) & 1][j] = TB::frag(sb, wn + j * 32, ks + 1, lane);
-        }
-#pragma unroll
-        for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[ks & 1][j], af[ks & 1][i], acc[i][j], 0, 0, 0);
-                const int q = ks * FM * FN + i * FN + j; // MFMA number within the stage
-                if (q < LOADS) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (copy)
-                        copy_one(q);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+        for (int i = 0; i < AF; ++i) {
+            f32x4 &t = acc[i >> 1][j >> 1][i & 1][j & 1];
+            t = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[column & 1], af[ks][i], t, 0, 0, 0);
+            const int q = column * AF + i; // instruction number within the stage
+            if ((q & 1) == 0 && q / 2 < LOADS) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (copy)
+                    copy_one(q / 2);
+                __builtin_amdgcn_sched_barrier(0);
             }
+        }
     }
 }
 
@@ -585,14 +670,14 @@ __global__ __launch_bounds__(256, 2) void gemm64_kernel(const bf16_t *__restrict
     for (int item = blockIdx.x; item < items; item += stride) {
         int m0, n0, c0, nc;
         const int split = locate(item, m0, n0, c0, nc);
-        f32x16 acc[FM][FN];
+        f32x4 acc[FM][FN][2][2]; // 32 x 32 blocks as 2 x 2 tiles of 16 x 16
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    acc[i][j][r] = 0.f;
+                for (int t = 0; t < 4; ++t)
+                    acc[i][j][t >> 1][t & 1] = f32x4{0.f, 0.f, 0.f, 0.f};
         u32x4 aux[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}}; // the epilogue's second input for tile (0, 0)
         for (int c = 0; c < nc; ++c) {
             wait_vmcnt<0>(); // this wave's copies of stage c (and the previous tile's stores) are done
@@ -744,14 +829,14 @@ __global__ __launch_bounds__(256, 2) void wgrad_batch_kernel(WgradBatch w) {
         WgradItem item;
         if (!wgrad_item(w, group, blockIdx.x, item))
             continue;
-        f32x16 acc[FM][FN];
+        f32x4 acc[FM][FN][2][2];
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    acc[i][j][r] = 0.f;
+                for (int t = 0; t < 4; ++t)
+                    acc[i][j][t >> 1][t & 1] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int c = 0; c < item.nc; ++c) {
             wait_vmcnt<0>();
             __syncthreads();
