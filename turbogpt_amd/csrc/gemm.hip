@@ -52,19 +52,19 @@ struct EpilogueBf16 {
         return *reinterpret_cast<const u32x4 *>(aux + size_t(m) * ld_aux + n);
     }
     // y: the bf16-rounded accumulators of row m, columns n .. n+7
-    TG_DEVICE void finish(int m, int n, u32x4 y, u32x4 a) const {
-        if (mode == EPI_RESIDUAL) {
+    template <int MODE> TG_DEVICE void finish_as(int m, int n, u32x4 y, u32x4 a) const {
+        if constexpr (MODE == EPI_RESIDUAL) {
             // RN(RN(acc) + residual): the bf16 add of cuda/mma.cuh:95-97
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 y[e] = pack_bf16(bf16_lo(y[e]) + bf16_lo(a[e]), bf16_hi(y[e]) + bf16_hi(a[e]));
-        } else if (mode == EPI_GELU_BWD) {
+        } else if constexpr (MODE == EPI_GELU_BWD) {
             // du = RN(RN(acc) * gelu'(u))
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 y[e] = pack_bf16(bf16_lo(y[e]) * gelu_grad_f(bf16_lo(a[e])),
                                  bf16_hi(y[e]) * gelu_grad_f(bf16_hi(a[e])));
-        } else if (mode == EPI_GELU) {
+        } else if constexpr (MODE == EPI_GELU) {
             u32x4 g;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -77,6 +77,27 @@ struct EpilogueBf16 {
         }
         *reinterpret_cast<u32x4 *>(out + size_t(m) * ld_out + n) = y;
     }
+    TG_DEVICE void finish(int m, int n, u32x4 y, u32x4 a) const {
+        if (mode == EPI_RESIDUAL)
+            finish_as<EPI_RESIDUAL>(m, n, y, a);
+        else if (mode == EPI_GELU_BWD)
+            finish_as<EPI_GELU_BWD>(m, n, y, a);
+        else if (mode == EPI_GELU)
+            finish_as<EPI_GELU>(m, n, y, a);
+        else
+            finish_as<EPI_PLAIN>(m, n, y, a);
+    }
+};
+// The same with the mode fixed at compile time.  A wave's loads and stores share one in-order counter, and a wait
+// names how many younger operations may stay outstanding: with the mode decided by branches that number is unknown
+// and every 32 x 32 block of the epilogue ends up waiting for its own stores to be acknowledged; with straight-line
+// code the stores of a block stay in flight while the next is rounded and transposed.
+template <int MODE> struct EpilogueBf16As {
+    static constexpr bool BF16 = true;
+    EpilogueBf16 any;
+    TG_DEVICE bool wants_aux() const { return MODE == EPI_RESIDUAL || MODE == EPI_GELU_BWD; }
+    TG_DEVICE u32x4 load_aux(int m, int n) const { return any.load_aux(m, n); }
+    TG_DEVICE void finish(int m, int n, u32x4 y, u32x4 a) const { any.finish_as<MODE>(m, n, y, a); }
 };
 
 // fp32 outputs (weight gradients, split-K slabs): tiles go through the same kind of wave-private LDS
@@ -182,6 +203,7 @@ TG_DEVICE void staged_store_bf16(const f32x4 (&acc)[FM][FN][2][2], const u32x4 (
     const int put_swizzle = (row >> 2) & 3, put_chunk = lane >> 5;
     const unsigned char *get = mine + get_row * 64 + ((get_chunk ^ ((get_row >> 2) & 3)) << 4);
     const bool wants_aux = epilogue.wants_aux();
+    // the second input is fetched one block ahead (two or more measured no faster, and cost registers)
     u32x4 aux[2] = {first[0], first[1]};
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -195,10 +217,10 @@ TG_DEVICE void staged_store_bf16(const f32x4 (&acc)[FM][FN][2][2], const u32x4 (
             for (int tm = 0; tm < 2; ++tm)
 #pragma unroll
                 for (int tn = 0; tn < 2; ++tn) {
-                    const f32x4 &t = acc[i][j][tm][tn];
+                    const f32x4 &tile = acc[i][j][tm][tn];
                     u32x2 packed;
-                    packed.x = pack_bf16(t[0], t[1]);
-                    packed.y = pack_bf16(t[2], t[3]);
+                    packed.x = pack_bf16(tile[0], tile[1]);
+                    packed.y = pack_bf16(tile[2], tile[3]);
                     *reinterpret_cast<u32x2 *>(put + tm * 1024 + (((2 * tn + put_chunk) ^ put_swizzle) << 4)) = packed;
                 }
             epilogue.finish(m, n, *reinterpret_cast<const u32x4 *>(get), aux[0]);
@@ -1062,6 +1084,22 @@ void launch_gemm64(hipStream_t stream, Tile tile, const bf16_t *A, int lda, cons
         launch_gemm64_tile<128, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
 }
 
+// bf16 epilogues of the 64-k kernel: one instantiation per mode
+template <bool AKC, bool BKC>
+void launch_gemm64_bf16(hipStream_t stream, Tile tile, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N,
+                        int K, const EpilogueBf16 &e) {
+    switch (e.mode) {
+    case EPI_RESIDUAL:
+        return launch_gemm64<AKC, BKC>(stream, tile, A, lda, B, ldb, M, N, K, 1, EpilogueBf16As<EPI_RESIDUAL>{e});
+    case EPI_GELU:
+        return launch_gemm64<AKC, BKC>(stream, tile, A, lda, B, ldb, M, N, K, 1, EpilogueBf16As<EPI_GELU>{e});
+    case EPI_GELU_BWD:
+        return launch_gemm64<AKC, BKC>(stream, tile, A, lda, B, ldb, M, N, K, 1, EpilogueBf16As<EPI_GELU_BWD>{e});
+    default:
+        return launch_gemm64<AKC, BKC>(stream, tile, A, lda, B, ldb, M, N, K, 1, EpilogueBf16As<EPI_PLAIN>{e});
+    }
+}
+
 void check_operand(const void *p, int ld, const char *name) {
     if (!p || (reinterpret_cast<uintptr_t>(p) & 15) || ld % 8)
         throw std::invalid_argument(std::string("gemm operand ") + name +
@@ -1100,7 +1138,7 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
             e.out2 = gelu_out, e.ld_out2 = ldg, e.mode = EPI_GELU;
         }
         if (takes_64(tile, K))
-            launch_gemm64<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, 1, e);
+            launch_gemm64_bf16<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, e);
         else
             dispatch_gemm<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, 1, e);
     });
@@ -1170,7 +1208,7 @@ extern "C" int tgk_gemm_dgrad_t(hipStream_t stream, int M, int N, int K, const u
         }
         // C[m][i] = sum_o dY[m][o] Wt[i][o]: the forward product with (rows, reduced) = (K, N)
         if (takes_64(tile, N))
-            launch_gemm64<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, 1, e);
+            launch_gemm64_bf16<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, e);
         else
             dispatch_gemm<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, 1, e);
     });
