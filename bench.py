@@ -294,9 +294,10 @@ def main():
         rate = amount / (per_step_ms * 1e-3) / 1e12 if per_step_ms > 0 else 0.0
         classes[name] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // 3,
                          ("tflops" if kind == "flop" else "tb_per_s"): round(rate, 2)}
-    # dominant MFMA kernel: gemm64_kernel<128,192,true,true,EpilogueBf16> - both operands contiguous along the
-    # reduced dimension - which runs the forward block projections (on the weights) and the dgrads (on their
-    # transposed copies): 8 launches per layer, 96 per step, the same four shapes in both directions.
+    # dominant MFMA kernel: gemm64_kernel<128,192,true,true,EpilogueBf16As<mode>> - both operands contiguous along
+    # the reduced dimension, one instantiation per epilogue (plain, + residual, GELU, GELU') - which runs the forward
+    # block projections (on the weights) and the dgrads (on their transposed copies): 8 launches per layer, 96 per
+    # step, the same four shapes in both directions.
     fwd_ms, fwd_launches = profile["gemm_fwd"]
     dgrad_ms, dgrad_launches = profile["gemm_dgrad"]
     launch_ms = (fwd_ms + dgrad_ms) / (fwd_launches + dgrad_launches)
@@ -321,8 +322,9 @@ def main():
                                "wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
                    "global_batch": B, "seq_len": T, "parameters": params, "parallelism": "single GPU"},
         "roofline": {"bound": "mfma",
-                     "kernel": "gemm64_kernel<128,192,true,true,EpilogueBf16> (forward block projections and "
-                               "dgrads: QKV, attention-out, MLP-up, MLP-down)",
+                     "kernel": "gemm64_kernel<128,192,true,true,EpilogueBf16As<mode>>, its four epilogue "
+                               "instantiations together (forward block projections and dgrads: QKV, attention-out, "
+                               "MLP-up, MLP-down)",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": hbm_traffic_per_launch(),
                      "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE of --traffic-probe, "
