@@ -191,10 +191,16 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_kernel(const bf16_t *__restri
     const int my_tiles = wave_q0 / 64 + 1; // tiles with a key visible to this wave (wave uniform)
     const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
     const uint32_t lds0 = lds_address(&stages[0][0][0]);
+    // a copy takes a wave-uniform tile address and a per-lane byte offset computed once: no vector arithmetic per tile
+    const uint32_t lane_offset[2] = {tile_copy_offset(ld, wave, lane, 0), tile_copy_offset(ld, wave, lane, 1)};
     auto produce = [&](int stage, int j) {
         const uint32_t slot = lds0 + uint32_t(stage) * (2 * TILE_ELEMS * 2);
-        tile_copy_async(slot, kbase + size_t(j) * 64 * ld, ld, wave, lane);
-        tile_copy_async(slot + TILE_ELEMS * 2, vbase + size_t(j) * 64 * ld, ld, wave, lane);
+        const bf16_t *kt = kbase + size_t(j) * 64 * ld, *vt = vbase + size_t(j) * 64 * ld;
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            async_copy16(__builtin_amdgcn_readfirstlane(slot + (wave + 4 * n) * 1024), kt, lane_offset[n]);
+            async_copy16(__builtin_amdgcn_readfirstlane(slot + TILE_ELEMS * 2 + (wave + 4 * n) * 1024), vt, lane_offset[n]);
+        }
     };
     produce(0, 0);
     if (tiles > 1)
@@ -458,10 +464,16 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
     const int my_tiles = wave_q0 / 64 + 1;
     const bf16_t *kbase = K + token0 * ld + h * HD, *vbase = V + token0 * ld + h * HD;
     const uint32_t lds0 = lds_address(&stages[0][0][0]);
+    // a copy takes a wave-uniform tile address and a per-lane byte offset computed once: no vector arithmetic per tile
+    const uint32_t lane_offset[2] = {tile_copy_offset(ld, wave, lane, 0), tile_copy_offset(ld, wave, lane, 1)};
     auto produce = [&](int stage, int j) {
         const uint32_t slot = lds0 + uint32_t(stage) * (2 * TILE_ELEMS * 2);
-        tile_copy_async(slot, kbase + size_t(j) * 64 * ld, ld, wave, lane);
-        tile_copy_async(slot + TILE_ELEMS * 2, vbase + size_t(j) * 64 * ld, ld, wave, lane);
+        const bf16_t *kt = kbase + size_t(j) * 64 * ld, *vt = vbase + size_t(j) * 64 * ld;
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            async_copy16(__builtin_amdgcn_readfirstlane(slot + (wave + 4 * n) * 1024), kt, lane_offset[n]);
+            async_copy16(__builtin_amdgcn_readfirstlane(slot + TILE_ELEMS * 2 + (wave + 4 * n) * 1024), vt, lane_offset[n]);
+        }
     };
     produce(0, 0);
     if (tiles > 1)
