@@ -316,7 +316,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
     const float *__restrict__ delta, bf16_t *__restrict__ dK, bf16_t *__restrict__ dV, int lddq, int T,
     int H, int pairs, float scale) {
     __shared__ __align__(1024) bf16_t stages[3][2][TILE_ELEMS]; // [stage][Q | dO]
-    __shared__ __align__(256) float rows[3][2][64];             // [stage][lse2 | delta]
+    __shared__ __align__(256) float rows[3][2][64];             // [stage][lse2 | -delta]
     const CausalBlock block = causal_block(H, pairs);
     if (!block.live)
         return;
@@ -381,7 +381,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
             const int qh = q0 + qt * 32;
             if (qh + 31 < wave_k0) // every query of this half precedes this wave's keys (wave uniform)
                 return;
-            f32x16 s = zero16(), dp = zero16();
+            // dP - delta in one go: the product accumulates onto -delta of its rows (the dQ kernel leaves the deltas
+            // negated), one subtraction per score less on the vector ALU that bounds this kernel
+            f32x16 s = zero16(), dp;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const f32x4 minus4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][1][qt * 32 + 8 * q4 + 4 * g]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    dp[q4 * 4 + e] = minus4[e];
+            }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 s = mfma(qrows.load(qt_tile, qt, ks), kf[ks], s);
@@ -394,7 +403,6 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
                 for (int q4 = 0; q4 < 4; ++q4) {
                     const int at = qt * 32 + 8 * q4 + 4 * g;
                     const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][0][at]);
-                    const f32x4 del4 = *reinterpret_cast<const f32x4 *>(&rows[STAGE][1][at]);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int r = q4 * 4 + e;
@@ -402,7 +410,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(
                         if (decltype(masked)::value && krow > q0 + at + e)
                             p = 0.f;
                         s[r] = p;
-                        dp[r] = p * (dp[r] - del4[e]);
+                        dp[r] = p * dp[r];
                     }
                 }
             };
@@ -506,7 +514,7 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
     const size_t row_at = (size_t(b) * H + h) * T + qrow;
     const float lse = LSE[row_at] * LOG2E;
     if (g == 0) {
-        delta_out[row_at] = del;
+        delta_out[row_at] = -del; // negated: the dK/dV kernel starts its dP product from it
         lse2_out[row_at] = lse;
     }
     f32x16 dq[2] = {zero16(), zero16()};
