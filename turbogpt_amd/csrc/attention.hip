@@ -518,6 +518,10 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
         lse2_out[row_at] = lse;
     }
     f32x16 dq[2] = {zero16(), zero16()};
+    f32x16 minus_delta;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        minus_delta[r] = -del;
     const RowFragOffsets krows(lane);
     const ColFragOffsets kcols(lane);
 
@@ -542,11 +546,12 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
         for (int mt = 0; mt < 2; ++mt) {
             if (kv0 + mt * 32 > wave_q0 + 31) // every key of this half follows this wave's queries
                 continue;
-            f32x16 s = zero16(), dp = zero16();
+            // dP - delta in one go: the product accumulates onto a register set that holds -delta of this lane's query
+            f32x16 s = zero16(), dp;
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 s = mfma(krows.load(kt, mt, ks), qf[ks], s);
-                dp = mfma(krows.load(vt, mt, ks), gf[ks], dp);
+                dp = mfma(krows.load(vt, mt, ks), gf[ks], ks == 0 ? minus_delta : dp);
             }
             // the causal mask only in the tiles that straddle the diagonal (wave-uniform branch)
             auto probabilities = [&](auto masked) {
@@ -555,7 +560,7 @@ __global__ __launch_bounds__(256, 3) void attn_bwd_dq_kernel(
                     float p = exp2_fast(fmaf(s[r], c, -lse));
                     if (decltype(masked)::value && kv0 + mt * 32 + acc_row(r, g) > qrow)
                         p = 0.f;
-                    dp[r] = p * (dp[r] - del);
+                    dp[r] = p * dp[r];
                 }
             };
             if (diagonal)
