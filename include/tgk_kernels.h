@@ -93,6 +93,23 @@ TGK_API int tgk_gemm_wgrad_batch(hipStream_t stream, int M, int count, const Tgk
                                  void *workspace, size_t workspace_bytes);
 TGK_API size_t tgk_gemm_wgrad_batch_workspace(int M, int count, const TgkWgradJob *jobs);
 
+/* Every weight gradient of a training step in one launch: any number of jobs (1..4096) that share the reduced
+ * dimension M, dW_j[N_j][K_j] = dY_j[M][N_j]^T . X_j[M][K_j], fp32, deterministic.  Takes the slot of all the
+ * weight_gradient calls of a backward pass (cuda/ops.cuh:83-109, called per matrix from cuda/model.cuh:61-99) and of
+ * reduce_gradients (cuda/trainer.cuh:9-47).  With several 256 x 256 output tiles per compute unit, all but the last
+ * (tiles mod compute units) tiles are reduced over all M rows by one block, in row order, and written once; the
+ * last ones are cut into row ranges whose partial sums a second launch adds in row order.  The caller keeps all
+ * operands alive until this call (the output gradients of every layer).  Every N_j and K_j a multiple of 256, M of
+ * 128, accumulate = 0.  The job and tile tables live in device memory: tgk_gemm_wgrad_list_prepare writes them into
+ * `table` (tgk_gemm_wgrad_list_table_bytes bytes, 16-byte aligned) with a synchronous copy, once per job list;
+ * tgk_gemm_wgrad_list is then called with the same M, jobs and table.  `workspace` holds
+ * tgk_gemm_wgrad_list_workspace bytes (may be NULL when that is 0). */
+TGK_API size_t tgk_gemm_wgrad_list_table_bytes(int M, int count, const TgkWgradJob *jobs);
+TGK_API size_t tgk_gemm_wgrad_list_workspace(int M, int count, const TgkWgradJob *jobs);
+TGK_API int tgk_gemm_wgrad_list_prepare(int M, int count, const TgkWgradJob *jobs, void *table, size_t table_bytes);
+TGK_API int tgk_gemm_wgrad_list(hipStream_t stream, int M, int count, const TgkWgradJob *jobs, const void *table,
+                                int accumulate, void *workspace, size_t workspace_bytes);
+
 
 /* ---- Causal softmax attention, head_dim 64.  Takes the slot of attention_forward /
  * attention_backward (cuda/attention.cuh:48-106); the reference's arg-max attention is replaced

@@ -229,6 +229,115 @@ def test_wgrad_batch_rejects_bad_jobs():
     sync()
 
 
+def run_wgrad_list(M, shapes, rng, strides=None):
+    """One tgk_gemm_wgrad_list over `shapes` (N, K); dW starts as NaN so an unwritten element shows."""
+    import ctypes as C
+    from turbogpt_amd.bridge import WgradJob
+    lib = library()
+    jobs = (WgradJob * len(shapes))()
+    keep, inputs = [], []
+    for j, (N, K) in enumerate(shapes):
+        extra = 0 if strides is None else strides[j]
+        dy, dyh = to_bf16_device(rng.standard_normal((M, N + extra)))
+        x, xh = to_bf16_device(rng.standard_normal((M, K + extra)))
+        dw = torch.full((N, K + extra), float("nan"), dtype=torch.float32, device="cuda")
+        keep.append((dy, x, dw))
+        inputs.append((np.ascontiguousarray(dyh[:, :N]), np.ascontiguousarray(xh[:, :K])))
+        jobs[j] = WgradJob(N, K, dy.data_ptr(), N + extra, x.data_ptr(), K + extra, dw.data_ptr(), K + extra)
+    table_bytes = lib.tgk_gemm_wgrad_list_table_bytes(M, len(shapes), C.addressof(jobs))
+    assert table_bytes > 0
+    table = torch.empty(table_bytes, dtype=torch.uint8, device="cuda")
+    need = lib.tgk_gemm_wgrad_list_workspace(M, len(shapes), C.addressof(jobs))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    check(lib.tgk_gemm_wgrad_list_prepare(M, len(shapes), C.addressof(jobs), table.data_ptr(), table_bytes))
+    call = lambda: check(lib.tgk_gemm_wgrad_list(stream(), M, len(shapes), C.addressof(jobs), table.data_ptr(), 0,
+                                                 ws.data_ptr(), need))
+    call()
+    sync()
+    return keep, inputs, (jobs, table, ws, call)
+
+
+@pytest.mark.parametrize("M,shapes", [(128, [(256, 256)]),                      # one tile, one quad
+                                      (512, [(768, 768)]),                      # fewer tiles than blocks: all split
+                                      (1024, [(256, 768), (768, 256), (512, 512)]),
+                                      (512, [(3072, 3072), (3072, 3072), (256, 768)]),  # whole tiles and split ones
+                                      (256, [(3072, 3072)] * 4),                # two whole tiles per block, then halves
+                                      (8192, [(768, 768)]),                     # long token ranges
+                                      (256, [(2304, 768), (768, 768), (3072, 768), (768, 3072)] * 3),
+                                      (384, [(1024, 4096), (4096, 1024), (1024, 1024), (3072, 1024), (256, 1024)])])
+def test_wgrad_list_against_the_checker(orc, M, shapes):
+    """All weight gradients of a step in one launch: every job against the checker, every element written, and a
+    second run bit-identical (whole tiles are summed in token order by one block, pieces in token-range order)."""
+    keep, inputs, (jobs, table, ws, call) = run_wgrad_list(M, shapes, np.random.default_rng(M + len(shapes)))
+    firsts = []
+    for (dy, x, dw), (dyh, xh) in zip(keep, inputs):
+        got = host(dw)
+        assert np.isfinite(got).all()
+        assert rel(got, orc.gemm_wgrad(dyh, xh)) < 1e-4
+        firsts.append(got.copy())
+        dw.fill_(float("nan"))
+    call()
+    sync()
+    for (dy, x, dw), first in zip(keep, firsts):
+        np.testing.assert_array_equal(host(dw), first)
+
+
+def test_wgrad_list_with_leading_dimensions(orc):
+    # operands and gradients that are column slices of wider buffers
+    shapes = [(512, 256), (256, 768)]
+    keep, inputs, _ = run_wgrad_list(256, shapes, np.random.default_rng(12), strides=[64, 8])
+    for (dy, x, dw), (dyh, xh), (N, K) in zip(keep, inputs, shapes):
+        got = host(dw)
+        assert rel(got[:, :K], orc.gemm_wgrad(dyh, xh)) < 1e-4
+        assert np.isnan(got[:, K:]).all()  # nothing written beside the gradient
+
+
+def test_wgrad_list_of_a_step_at_full_size(orc):
+    """A block's four weight gradients at M = 16384 (config 2's shapes), three blocks' worth plus the head's, in one
+    launch: against one tgk_gemm_wgrad per matrix (fp32 sums in a different order: 1e-5) and the checker on sampled
+    rows of every matrix."""
+    lib = library()
+    M = 16384
+    shapes = [(768, 3072), (3072, 768), (768, 768), (2304, 768)] * 3 + [(256, 768)]
+    rng = np.random.default_rng(77)
+    keep, inputs, _ = run_wgrad_list(M, shapes, rng)
+    for (dy, x, dw), (dyh, xh), (N, K) in zip(keep, inputs, shapes):
+        need = lib.tgk_gemm_wgrad_workspace(M, N, K)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        single = torch.empty(N, K, dtype=torch.float32, device="cuda")
+        check(lib.tgk_gemm_wgrad(stream(), M, N, K, dy.data_ptr(), N, x.data_ptr(), K, single.data_ptr(), K, 0,
+                                 ws.data_ptr(), need))
+        sync()
+        assert rel(host(dw), host(single)) < 1e-5
+        cols = np.sort(rng.choice(N, 8, replace=False))
+        assert rel(host(dw)[cols], orc.gemm_wgrad(np.ascontiguousarray(dyh[:, cols]), xh)) < 1e-4
+
+
+def test_wgrad_list_rejects_bad_jobs():
+    import ctypes as C
+    from turbogpt_amd.bridge import WgradJob
+    lib = library()
+    t = torch.zeros(256 * 256, dtype=torch.bfloat16, device="cuda")
+    f = torch.zeros(256 * 256, dtype=torch.float32, device="cuda")
+    jobs = (WgradJob * 1)(WgradJob(256, 192, t.data_ptr(), 256, t.data_ptr(), 192, f.data_ptr(), 192))
+    assert lib.tgk_gemm_wgrad_list_table_bytes(128, 1, C.addressof(jobs)) == 0
+    assert lib.tgk_gemm_wgrad_list_prepare(128, 1, C.addressof(jobs), f.data_ptr(), 1 << 16) == -1
+    assert b"multiple of 256" in lib.tgk_error()
+    jobs[0].K = jobs[0].ldx = jobs[0].lddw = 256
+    bytes_needed = lib.tgk_gemm_wgrad_list_table_bytes(128, 1, C.addressof(jobs))
+    assert bytes_needed > 0
+    assert lib.tgk_gemm_wgrad_list_table_bytes(64, 1, C.addressof(jobs)) == 0  # M % 128
+    assert lib.tgk_gemm_wgrad_list_prepare(128, 1, C.addressof(jobs), f.data_ptr(), bytes_needed - 1) == -1
+    assert b"table too small" in lib.tgk_error()
+    check(lib.tgk_gemm_wgrad_list_prepare(128, 1, C.addressof(jobs), f.data_ptr(), 1 << 16))
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    assert lib.tgk_gemm_wgrad_list(stream(), 128, 1, C.addressof(jobs), f.data_ptr(), 1, ws.data_ptr(), 1 << 20) == -1
+    assert b"accumulate" in lib.tgk_error()
+    assert lib.tgk_gemm_wgrad_list(stream(), 128, 1, C.addressof(jobs), None, 0, ws.data_ptr(), 1 << 20) == -1
+    assert lib.tgk_gemm_wgrad_list(stream(), 128, 0, C.addressof(jobs), f.data_ptr(), 0, ws.data_ptr(), 1 << 20) == -1
+    sync()
+
+
 def test_strided_views_of_a_packed_buffer(orc):
     # the engine hands out column slices of wider buffers: leading dimensions differ from widths
     lib = library()

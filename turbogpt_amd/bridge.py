@@ -25,6 +25,10 @@ KERNEL_ABI = {
     "tgk_gemm_wgrad_workspace": (sz, [i32, i32, i32]),
     "tgk_gemm_wgrad_batch": (i32, [vp, i32, i32, vp, i32, vp, sz]),
     "tgk_gemm_wgrad_batch_workspace": (sz, [i32, i32, vp]),
+    "tgk_gemm_wgrad_list_table_bytes": (sz, [i32, i32, vp]),
+    "tgk_gemm_wgrad_list_workspace": (sz, [i32, i32, vp]),
+    "tgk_gemm_wgrad_list_prepare": (i32, [i32, i32, vp, vp, sz]),
+    "tgk_gemm_wgrad_list": (i32, [vp, i32, i32, vp, vp, i32, vp, sz]),
     "tgk_attn_fwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, f32]),
     "tgk_attn_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32,
                            f32, vp, sz]),

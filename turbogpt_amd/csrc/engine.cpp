@@ -70,6 +70,12 @@ struct Slot {
     std::vector<LayerBuffers> layers;
     bf16_t *nf = nullptr, *logits = nullptr, *dh = nullptr, *t1 = nullptr, *du = nullptr, *dqkv = nullptr;
     bf16_t *dh_mid = nullptr; // the gradient between a block's two halves, when the block's weight gradients are batched
+    // When all weight gradients of a step go out as one launch behind the backward pass, every block keeps the four
+    // output gradients that launch reads: g_x[l] = gradient of the loss by x[l] (g_x[l + 1] enters block l), g_mid[l]
+    // by the block's middle, g_u[l] by the MLP pre-activation, g_qkv[l] by the packed projections.
+    std::vector<bf16_t *> g_x, g_mid, g_u, g_qkv;
+    std::vector<TgkWgradJob> wgrad_jobs;
+    void *wgrad_table = nullptr;
     void *workspace = nullptr;
     // LayerNorm parameter gradients: every LayerNorm backward of a step leaves its per-block partial sums in a
     // block of its own here and one launch at the end of the backward pass folds all 2 * depth + 1 of them
@@ -107,6 +113,7 @@ struct Engine {
     float *logits_f32 = nullptr;
     size_t workspace_bytes = 0;
     bool batched_wgrad = false; // a block's four weight gradients in one launch (shapes permitting)
+    bool list_wgrad = false;    // every weight gradient of a step in one launch (widths that are multiples of 256)
 
     std::vector<StepRates> schedule;
     uint64_t step = 0;
@@ -274,8 +281,6 @@ struct Engine {
         const int M = tokens(), d = config.d_model, F = config.ffn, V = config.vocab, T = c.context;
         const float scale = 1.0f / std::sqrt(float(d / config.heads));
         float *g = gradient;
-        OP(TG_CLASS_HEAD, tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
-        OP(TG_CLASS_HEAD, tgk_gemm_dgrad_t(stream, M, V, d, logits, V, wt(layout.head), V, t1, d, nullptr, 0));
         // LayerNorm j of the fold: 0 = final, 1 + 2 l = block l's second, 2 + 2 l = its first
         const size_t ln_stride = tgk_layernorm_bwd_workspace(M, d);
         const auto ln_rows = [&](int job, const bf16_t *input, const bf16_t *dy, int64_t gamma, const bf16_t *residual,
@@ -283,6 +288,35 @@ struct Engine {
             return tgk_layernorm_bwd_rows(stream, M, d, input, dy, w(gamma), wl(gamma), residual, dx, config.ln_eps,
                                           s.ln_partials + size_t(job) * ln_stride, ln_stride);
         };
+        if (list_wgrad) {
+            // No weight gradient in the loop: every block leaves its output gradients in buffers of its own and one
+            // launch at the end computes all 4 * depth + 1 products (the head's included; its operands are dlogits,
+            // still in `logits`, and nf).
+            OP(TG_CLASS_HEAD, tgk_gemm_dgrad_t(stream, M, V, d, logits, V, wt(layout.head), V, t1, d, nullptr, 0));
+            OP(TG_CLASS_LAYERNORM_BWD, ln_rows(0, x[c.depth], t1, layout.lnf_g, nullptr, s.g_x[c.depth]));
+            for (int l = c.depth - 1; l >= 0; --l) {
+                const TgLayerParameters &p = layout.layers[l];
+                LayerBuffers &b = layers[l];
+                bf16_t *in = s.g_x[l + 1], *mid = s.g_mid[l], *gu = s.g_u[l], *gqkv = s.g_qkv[l];
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, in, d, wt(p.mlp_down), d, gu, F, b.u, F));
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, gu, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
+                OP(TG_CLASS_LAYERNORM_BWD, ln_rows(1 + 2 * l, b.mid, t1, p.ln2_g, in, mid));
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, d, mid, d, wt(p.attn_out), d, t1, d, nullptr, 0));
+                OP(TG_CLASS_ATTN_BWD, tgk_attn_bwd(stream, c.batch, config.heads, T, d / config.heads, b.qkv, b.qkv + d,
+                                                   b.qkv + 2 * d, 3 * d, b.o, d, b.lse, t1, d, gqkv, gqkv + d, gqkv + 2 * d,
+                                                   3 * d, scale, workspace, workspace_bytes));
+                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, 3 * d, d, gqkv, 3 * d, wt(p.qkv), 3 * d, t1, d, nullptr, 0));
+                OP(TG_CLASS_LAYERNORM_BWD, ln_rows(2 + 2 * l, x[l], t1, p.ln1_g, mid, s.g_x[l]));
+            }
+            OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_fold(stream, M, d, 2 * c.depth + 1, s.ln_partials, ln_stride, s.ln_targets, 0));
+            OP(TG_CLASS_OTHER, tgk_embed_bwd(stream, c.batch, T, d, V, tokens_in, s.g_x[0], g + layout.embedding,
+                                             g + layout.positions, 0, workspace, workspace_bytes));
+            OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad_list(stream, M, int(s.wgrad_jobs.size()), s.wgrad_jobs.data(), s.wgrad_table, 0,
+                                                        workspace, workspace_bytes));
+            return;
+        }
+        OP(TG_CLASS_HEAD, tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
+        OP(TG_CLASS_HEAD, tgk_gemm_dgrad_t(stream, M, V, d, logits, V, wt(layout.head), V, t1, d, nullptr, 0));
         OP(TG_CLASS_LAYERNORM_BWD, ln_rows(0, x[c.depth], t1, layout.lnf_g, nullptr, dh));
         for (int l = c.depth - 1; l >= 0; --l) {
             const TgLayerParameters &p = layout.layers[l];
@@ -663,8 +697,47 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
                                            {int(F), int(d), nullptr, int(F), nullptr, int(d), nullptr, int(d)},
                                            {int(d), int(d), nullptr, int(d), nullptr, int(d), nullptr, int(d)},
                                            {int(3 * d), int(d), nullptr, int(3 * d), nullptr, int(d), nullptr, int(d)}};
-        const size_t batch_need = tgk_gemm_wgrad_batch_workspace(int(M), 4, block_jobs);
-        e->batched_wgrad = batch_need > 0;
+        size_t batch_need = tgk_gemm_wgrad_batch_workspace(int(M), 4, block_jobs);
+        // One launch for all weight gradients where the shapes allow it (every width a multiple of 256)
+        size_t table_bytes = 0;
+        for (Slot &slot : e->slots) {
+            std::vector<TgkWgradJob> &jobs = slot.wgrad_jobs;
+            for (int l = 0; l < c.depth; ++l)
+                for (int j = 0; j < 4; ++j)
+                    jobs.push_back(block_jobs[j]);
+            jobs.push_back({int(V), int(d), nullptr, int(V), nullptr, int(d), nullptr, int(d)});
+            table_bytes = tgk_gemm_wgrad_list_table_bytes(int(M), int(jobs.size()), jobs.data());
+        }
+        e->list_wgrad = table_bytes > 0;
+        if (e->list_wgrad) {
+            batch_need = 0;
+            for (Slot &slot : e->slots) {
+                slot.g_x.resize(c.depth + 1), slot.g_mid.resize(c.depth), slot.g_u.resize(c.depth), slot.g_qkv.resize(c.depth);
+                for (int l = 0; l <= c.depth; ++l)
+                    e->allocate(slot.g_x[l], M * d, false);
+                for (int l = 0; l < c.depth; ++l) {
+                    e->allocate(slot.g_mid[l], M * d, false);
+                    e->allocate(slot.g_u[l], M * F, false);
+                    e->allocate(slot.g_qkv[l], M * 3 * d, false);
+                    const TgLayerParameters &p = e->layout.layers[l];
+                    const LayerBuffers &b = slot.layers[l];
+                    float *g = slot.gradient;
+                    TgkWgradJob *jobs = slot.wgrad_jobs.data() + 4 * l;
+                    jobs[0].dY = slot.g_x[l + 1], jobs[0].X = b.a, jobs[0].dW = g + p.mlp_down;
+                    jobs[1].dY = slot.g_u[l], jobs[1].X = b.n2, jobs[1].dW = g + p.mlp_up;
+                    jobs[2].dY = slot.g_mid[l], jobs[2].X = b.o, jobs[2].dW = g + p.attn_out;
+                    jobs[3].dY = slot.g_qkv[l], jobs[3].X = b.n1, jobs[3].dW = g + p.qkv;
+                }
+                TgkWgradJob &head = slot.wgrad_jobs.back();
+                head.dY = slot.logits, head.X = slot.nf, head.dW = slot.gradient + e->layout.head;
+                uint8_t *table = nullptr;
+                e->allocate(table, table_bytes, false);
+                slot.wgrad_table = table;
+                ok(tgk_gemm_wgrad_list_prepare(int(M), int(slot.wgrad_jobs.size()), slot.wgrad_jobs.data(), table, table_bytes));
+                batch_need = std::max(batch_need, tgk_gemm_wgrad_list_workspace(int(M), int(slot.wgrad_jobs.size()), slot.wgrad_jobs.data()));
+            }
+        }
+        e->batched_wgrad = !e->list_wgrad && batch_need > 0;
         if (e->batched_wgrad)
             for (Slot &slot : e->slots)
                 e->allocate(slot.dh_mid, M * d, false);

@@ -26,6 +26,8 @@
 // gradients of several matrices in one launch).
 #include "common.h"
 #include <atomic>
+#include <type_traits>
+#include <vector>
 #include "../../include/tgk_kernels.h"
 
 namespace {
@@ -934,6 +936,280 @@ __global__ __launch_bounds__(256) void wgrad_batch_fold_kernel(WgradBatch w) {
     }
 }
 
+// ---- every weight gradient of a step in one launch: 256-row tiles, one wave per SIMD ------------------------
+// dW_j[N_j][K_j] = dY_j^T X_j for any number of (dY, X) pairs that share the reduced dimension (the tokens).  A
+// training step has 4 * depth + 2 of them; taken together they have several tiles per compute unit, so almost every
+// tile is reduced over all tokens by one block (no partial sums, no fold) and only the last tiles % blocks tiles are
+// cut into token ranges.  The operands of all layers must exist at once: the caller keeps every layer's output
+// gradients until the end of the backward pass (a few GB of the 288).
+//
+// One block of four waves per compute unit, a 256 x BN tile, each wave 128 x BN/2 outputs (accumulators in 256
+// registers: a wave owns its SIMD's whole register file).  Per 32 k a wave then reads 16 KB of fragments for 64
+// matrix instructions where the 64 x 96 wave tile of gemm64_kernel reads 10 KB for 24, and the block copies 32 KB
+// per 4.2 MFLOP where two 128 x 192 blocks copy 40 KB for 3.1: less of everything that is not a matrix instruction
+// per flop, which is what the power limit pays for.  With one wave per SIMD nothing else covers a wave's waits, so:
+// a ring of four 32-k stages filled three stages ahead (a copy has three stages of matrix instructions to land), the
+// fragments of the next stage read into a second register set between the matrix instructions of the current one
+// (its data is published one stage early), one barrier per stage, and copies and fragment reads spread evenly
+// between the matrix instructions.
+struct WgradListJob {
+    const bf16_t *dy, *x;
+    float *dw;
+    int lddy, ldx, lddw, pad;
+};
+struct WgradList {
+    const WgradListJob *jobs; // device memory
+    const int4 *tiles;        // device memory: {job, first row, first column, 0} per tile, in processing order
+    int rounds;               // whole tiles per block
+    int rem_tiles, rem_splits; // the tiles after rounds * blocks, each cut into rem_splits token ranges
+    int k_quads;              // tokens / 128
+    int accumulate;
+    float *pieces; // rem_tiles * rem_splits partial tiles of 256 * BN floats, row major
+};
+struct WgradListItem {
+    int tile, q0, nq, piece; // piece < 0: the block reduces over all tokens and writes the gradient itself
+};
+// The i-th work item of this block.  Consecutive block ids sit on consecutive XCDs; an XCD takes 1/8 of the blocks'
+// consecutive tiles in every round, which are neighbours in one job's tile grid and walk the tokens together, so the
+// operand panels they share are read into that XCD's L2 once.
+TG_DEVICE bool wgrad_list_item(const WgradList &w, int i, WgradListItem &item) {
+    const int blocks = gridDim.x, b = blockIdx.x;
+    const int logical = (blocks & 7) == 0 ? (b & 7) * (blocks >> 3) + (b >> 3) : b;
+    if (i < w.rounds) {
+        item = {i * blocks + logical, 0, w.k_quads, -1};
+        return true;
+    }
+    if (i > w.rounds || logical >= w.rem_tiles * w.rem_splits)
+        return false;
+    const int split = logical / w.rem_tiles, r = logical - split * w.rem_tiles;
+    item.tile = w.rounds * blocks + r;
+    item.q0 = int(int64_t(split) * w.k_quads / w.rem_splits);
+    item.nq = int(int64_t(split + 1) * w.k_quads / w.rem_splits) - item.q0;
+    item.piece = w.rem_splits > 1 ? r * w.rem_splits + split : -1;
+    return true;
+}
+TG_DEVICE const char *uniform_pointer(const void *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(uint32_t(v)), hi = __builtin_amdgcn_readfirstlane(uint32_t(v >> 32));
+    return reinterpret_cast<const char *>(uint64_t(hi) << 32 | lo);
+}
+template <int ROWS> TG_DEVICE uint32_t ks_frag16_offset(int row0, int lane) { // TileKS<ROWS>::frag16's first address, k0 = 0
+    const int g = lane >> 4, i = lane & 15;
+    const int r = 8 * g + (i >> 2), col = row0 + 4 * (i & 3);
+    return uint32_t(r * (ROWS * 2) + (i & 1) * 8 + (((col >> 3) ^ TileKS<ROWS>::swizzle(r)) << 4));
+}
+template <int ROWS> TG_DEVICE bf16x8 ks_frag16_at(const unsigned char *p) { // k-rows r and r + 4 share a swizzle term
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * ROWS * 2));
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, both);
+}
+template <int BN>
+__global__ __launch_bounds__(256, 1) void wgrad_list_kernel(const WgradList w) {
+    constexpr int BM = 256, S = 4;
+    using TA = TileKS<BM>;
+    using TB = TileKS<BN>;
+    constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32, AF = 2 * FM, BF = 2 * FN, MFMAS = AF * BF;
+    constexpr int LA = TA::LOADS, LB = TB::LOADS, LOADS = LA + LB;
+    constexpr int A_RING = S * TA::BYTES;
+#ifndef WL_READ_EVERY
+#define WL_READ_EVERY 3
+#endif
+#ifndef WL_COPY_EVERY
+#define WL_COPY_EVERY (MFMAS / LOADS)
+#endif
+#ifndef WL_COPY_FIRST
+#define WL_COPY_FIRST 1
+#endif
+    constexpr int READ_EVERY = WL_READ_EVERY, COPY_EVERY = WL_COPY_EVERY, COPY_FIRST = WL_COPY_FIRST;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t smem_base = lds_address(smem);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+
+    // ---- producer: one quad (four stages) ahead of the consumer, across item boundaries -----------------------
+    int p_index = 0, p_left = 0;
+    const char *p_a = nullptr, *p_b = nullptr; // wave-uniform: the operands' first k-row of the stage to copy next
+    int64_t a_step = 0, b_step = 0;
+    uint32_t la[LA], lb[LB]; // this lane's byte offset inside a stage, per copy
+    auto producer_open = [&]() {
+        WgradListItem item;
+        if (!wgrad_list_item(w, p_index, item)) {
+            // Out of work: the copies go on (the loop below is straight-line code), re-reading the last stage into
+            // slots nobody consumes.
+            p_a -= a_step, p_b -= b_step;
+            a_step = b_step = 0;
+            p_left = 1 << 30;
+            return;
+        }
+        ++p_index;
+        const int4 t = w.tiles[item.tile];
+        const WgradListJob job = w.jobs[t.x];
+        // the tables are read with vector loads: tell the compiler that the values are the same in every lane
+        const int lddy = __builtin_amdgcn_readfirstlane(job.lddy), ldx = __builtin_amdgcn_readfirstlane(job.ldx);
+        p_left = __builtin_amdgcn_readfirstlane(item.nq * 4);
+        p_a = uniform_pointer(job.dy + int64_t(item.q0) * 128 * job.lddy + t.y);
+        p_b = uniform_pointer(job.x + int64_t(item.q0) * 128 * job.ldx + t.z);
+        a_step = int64_t(BK) * lddy * 2, b_step = int64_t(BK) * ldx * 2;
+#pragma unroll
+        for (int j = 0; j < LA; ++j)
+            la[j] = uint32_t(TA::source_offset(j, tid, job.lddy) * 2);
+#pragma unroll
+        for (int j = 0; j < LB; ++j)
+            lb[j] = uint32_t(TB::source_offset(j, tid, job.ldx) * 2);
+    };
+    auto copy_one = [&](int n, int slot) __attribute__((always_inline)) { // n-th of the LOADS copies of a stage
+        if (n < LA)
+            async_copy16(smem_base + uint32_t(slot * TA::BYTES + (n * 4 + wave) * 1024), p_a, la[n]);
+        else
+            async_copy16(smem_base + uint32_t(A_RING + slot * TB::BYTES + ((n - LA) * 4 + wave) * 1024), p_b, lb[n - LA]);
+    };
+    {
+        WgradListItem first;
+        if (!wgrad_list_item(w, 0, first))
+            return;
+    }
+    producer_open();
+#pragma unroll
+    for (int s = 0; s < S; ++s) { // every item is a whole number of quads
+#pragma unroll
+        for (int n = 0; n < LOADS; ++n)
+            copy_one(n, s);
+        p_a += a_step, p_b += b_step;
+    }
+    if ((p_left -= S) == 0)
+        producer_open();
+
+    // ---- consumer -------------------------------------------------------------------------------------------
+    uint32_t fa_at[AF], fb_at[BF]; // this lane's fragment addresses inside a stage
+#pragma unroll
+    for (int i = 0; i < AF; ++i)
+        fa_at[i] = ks_frag16_offset<BM>(wm + i * 16, lane);
+#pragma unroll
+    for (int j = 0; j < BF; ++j)
+        fb_at[j] = A_RING + ks_frag16_offset<BN>(wn + j * 16, lane);
+    auto read_fragment = [&](bf16x8 (&fa)[AF], bf16x8 (&fb)[BF], int slot, int f) __attribute__((always_inline)) {
+        if (f < AF)
+            fa[f] = ks_frag16_at<BM>(smem + fa_at[f] + slot * TA::BYTES);
+        else
+            fb[f - AF] = ks_frag16_at<BN>(smem + fb_at[f - AF] + slot * TB::BYTES);
+    };
+    f32x4 acc[FM][FN][2][2];
+    // Stage t's fragments are in `cur`; the step publishes stage t + 1, reads its fragments into `next` and copies
+    // stage t + 4 into the slot stage t leaves.  Straight-line code: no branch between the matrix instructions.
+    auto step = [&](auto slot_tag, const bf16x8 (&cur_a)[AF], const bf16x8 (&cur_b)[BF], bf16x8 (&next_a)[AF],
+                    bf16x8 (&next_b)[BF]) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_tag)::value, NEXT = (SLOT + 1) % S;
+        wait_vmcnt<(S - 2) * LOADS>(); // stages t + 2 and t + 3 may still be in flight
+        __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's reads of stage t are done, its slot may be overwritten
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < BF; ++j)
+#pragma unroll
+            for (int i = 0; i < AF; ++i) {
+                // the accumulators fill the accumulation registers exactly, the fragments live in the other 256: left to
+                // itself the register allocator mixes the two and spends the loop moving tiles between them
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                             : "+a"(acc[i >> 1][j >> 1][i & 1][j & 1])
+                             : "v"(cur_b[j]), "v"(cur_a[i]));
+                const int q = j * AF + i;
+#ifndef WL_NO_READ
+                if (q % READ_EVERY == 0 && q / READ_EVERY < AF + BF)
+                    read_fragment(next_a, next_b, NEXT, q / READ_EVERY);
+#endif
+#ifndef WL_NO_COPY
+                if (q >= COPY_FIRST && (q - COPY_FIRST) % COPY_EVERY == 0 && (q - COPY_FIRST) / COPY_EVERY < LOADS)
+                    copy_one((q - COPY_FIRST) / COPY_EVERY, SLOT);
+#endif
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        p_a += a_step, p_b += b_step;
+    };
+    bf16x8 fa0[AF], fb0[BF], fa1[AF], fb1[BF];
+    wait_vmcnt<(S - 1) * LOADS>(); // stage 0
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int f = 0; f < AF + BF; ++f)
+        read_fragment(fa0, fb0, 0, f);
+    // Zeroed by the matrix pipe (0 x 0 + 0), in place: an assignment would start a new value in other registers and
+    // the allocator would move all 256 into place inside the loop.  64 instructions per 32768.
+    const bf16x8 zeros = {0, 0, 0, 0, 0, 0, 0, 0};
+    auto clear = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    // The compiler does not know that this is a matrix instruction and leaves no wait states between
+                    // the moves that fill `zeros` and the instruction, which then multiplies what the registers held
+                    // before: the wait states are part of the statement.
+                    asm volatile("s_nop 4\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %1, 0"
+                                 : "+a"(acc[i][j][t >> 1][t & 1])
+                                 : "v"(zeros));
+    };
+    // One loop over the quads of all items: the accumulators are carried by a single loop, and an item's end is a
+    // (wave-uniform) branch behind the four steps.
+    WgradListItem item;
+    int index = 0;
+    wgrad_list_item(w, 0, item);
+    int quads_left = item.nq;
+    clear();
+    for (;;) {
+        step(std::integral_constant<int, 0>{}, fa0, fb0, fa1, fb1);
+        step(std::integral_constant<int, 1>{}, fa1, fb1, fa0, fb0);
+        step(std::integral_constant<int, 2>{}, fa0, fb0, fa1, fb1);
+        step(std::integral_constant<int, 3>{}, fa1, fb1, fa0, fb0);
+        if ((p_left -= S) == 0)
+            producer_open();
+        if (--quads_left)
+            continue;
+        // A lane holds 4 consecutive columns of one row per 16 x 16 tile: 16 rows x 64 bytes per store.  One running
+        // pointer, hidden from the optimiser between rows: 64 precomputed addresses would not fit beside the fragments.
+        const int4 t = w.tiles[item.tile];
+        const WgradListJob job = w.jobs[t.x];
+        float *out = item.piece < 0 ? job.dw + size_t(t.y) * job.lddw + t.z : w.pieces + size_t(item.piece) * (BM * BN);
+        const int ld = item.piece < 0 ? job.lddw : BN;
+        out += size_t(wm + (lane & 15)) * ld + wn + 4 * (lane >> 4);
+#pragma unroll
+        for (int i = 0; i < AF; ++i) {
+#pragma unroll
+            for (int j = 0; j < BF; ++j)
+                *reinterpret_cast<f32x4 *>(out + j * 16) = acc[i >> 1][j >> 1][i & 1][j & 1];
+            out += size_t(16) * ld;
+            asm volatile("" : "+v"(out));
+        }
+        // the copy counter must hold nothing but the three stages the steps assume: let the stores drain
+        wait_vmcnt<0>();
+        if (!wgrad_list_item(w, ++index, item))
+            break;
+        quads_left = item.nq;
+        clear();
+    }
+    wait_vmcnt<0>();
+}
+// Sums the pieces of the split tiles, in token order, into the gradient.  Eight blocks per tile.
+template <int BN> __global__ __launch_bounds__(256) void wgrad_list_fold_kernel(const WgradList w, int first_tile) {
+    constexpr int BM = 256, QUADS = BM * BN / 4 / 8 / 256; // float4 per thread
+    const int r = blockIdx.x >> 3, part = blockIdx.x & 7;
+    const int4 t = w.tiles[first_tile + r];
+    const WgradListJob job = w.jobs[t.x];
+    const float *first = w.pieces + size_t(r) * w.rem_splits * (BM * BN);
+#pragma unroll
+    for (int k = 0; k < QUADS; ++k) {
+        const int quad = (part * QUADS + k) * 256 + threadIdx.x;
+        const int row = quad / (BN / 4), col = (quad % (BN / 4)) * 4;
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int split = 0; split < w.rem_splits; ++split) // fixed order
+            sum += *reinterpret_cast<const f32x4 *>(first + size_t(split) * (BM * BN) + size_t(quad) * 4);
+        f32x4 *p = reinterpret_cast<f32x4 *>(job.dw + size_t(t.y + row) * job.lddw + t.z + col);
+        if (w.accumulate)
+            sum += *p;
+        __builtin_nontemporal_store(sum, p);
+    }
+}
+
 // Sums split-K slabs in a fixed order (deterministic) into the fp32 gradient.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ slabs,
                                                             size_t slab_stride, int splits,
@@ -1361,5 +1637,126 @@ extern "C" int tgk_gemm_wgrad_batch(hipStream_t stream, int M, int count, const 
         check_hip(hipGetLastError(), "wgrad batch launch: ");
         hipLaunchKernelGGL((wgrad_batch_fold_kernel<128, 192>), dim3(w.first_tile[count] * 4), dim3(256), 0, stream, w);
         check_hip(hipGetLastError(), "wgrad batch fold launch: ");
+    });
+}
+
+namespace {
+// Tables and split of a whole-step weight-gradient launch.
+struct WgradListPlan {
+    int tiles, blocks, rounds, rem_tiles, rem_splits;
+    size_t jobs_bytes, table_bytes, pieces_bytes;
+};
+bool plan_wgrad_list(int M, int count, const TgkWgradJob *jobs, WgradListPlan &plan, std::string &why) {
+    if (count < 1 || count > 4096 || !jobs) {
+        why = "gemm_wgrad_list: between 1 and 4096 jobs";
+        return false;
+    }
+    if (M <= 0 || M % 128) {
+        why = "gemm_wgrad_list: M (the reduced dimension) must be a multiple of 128";
+        return false;
+    }
+    int tiles = 0;
+    for (int j = 0; j < count; ++j) {
+        if (jobs[j].N <= 0 || jobs[j].K <= 0 || jobs[j].N % 256 || jobs[j].K % 256) {
+            why = "gemm_wgrad_list: every N and K must be a multiple of 256";
+            return false;
+        }
+        tiles += (jobs[j].N / 256) * (jobs[j].K / 256);
+    }
+    plan.tiles = tiles;
+    plan.blocks = compute_units();
+    plan.rounds = tiles / plan.blocks;
+    plan.rem_tiles = tiles % plan.blocks;
+    const int k_quads = M / 128;
+    plan.rem_splits = plan.rem_tiles ? std::min(plan.blocks / plan.rem_tiles, k_quads) : 1;
+    plan.jobs_bytes = (size_t(count) * sizeof(WgradListJob) + 15) / 16 * 16;
+    plan.table_bytes = plan.jobs_bytes + size_t(tiles) * sizeof(int4);
+    plan.pieces_bytes = plan.rem_splits > 1 ? size_t(plan.rem_tiles) * plan.rem_splits * 256 * 256 * sizeof(float) : 0;
+    return true;
+}
+} // namespace
+
+extern "C" size_t tgk_gemm_wgrad_list_table_bytes(int M, int count, const TgkWgradJob *jobs) {
+    try {
+        WgradListPlan plan;
+        std::string why;
+        return plan_wgrad_list(M, count, jobs, plan, why) ? plan.table_bytes : 0;
+    } catch (...) {
+        return 0;
+    }
+}
+extern "C" size_t tgk_gemm_wgrad_list_workspace(int M, int count, const TgkWgradJob *jobs) {
+    try {
+        WgradListPlan plan;
+        std::string why;
+        return plan_wgrad_list(M, count, jobs, plan, why) ? plan.pieces_bytes : 0;
+    } catch (...) {
+        return 0;
+    }
+}
+extern "C" int tgk_gemm_wgrad_list_prepare(int M, int count, const TgkWgradJob *jobs, void *table, size_t table_bytes) {
+    return guarded([&] {
+        WgradListPlan plan;
+        std::string why;
+        if (!plan_wgrad_list(M, count, jobs, plan, why))
+            throw std::invalid_argument(why);
+        require(table && table_bytes >= plan.table_bytes && !(reinterpret_cast<uintptr_t>(table) & 15),
+                "gemm_wgrad_list_prepare: table too small (see tgk_gemm_wgrad_list_table_bytes)");
+        std::vector<unsigned char> host(plan.table_bytes, 0);
+        WgradListJob *job_table = reinterpret_cast<WgradListJob *>(host.data());
+        int4 *tile_table = reinterpret_cast<int4 *>(host.data() + plan.jobs_bytes);
+        int tile = 0;
+        for (int j = 0; j < count; ++j) {
+            const TgkWgradJob &job = jobs[j];
+            check_operand(job.dY, job.lddy, "dY");
+            check_operand(job.X, job.ldx, "X");
+            require(job.lddy >= job.N && job.ldx >= job.K, "gemm_wgrad_list: leading dimension too small");
+            require(job.dW && !(reinterpret_cast<uintptr_t>(job.dW) & 15) && job.lddw % 4 == 0 && job.lddw >= job.K,
+                    "gemm_wgrad_list: dW must be 16-byte aligned with leading dimension % 4 == 0");
+            job_table[j] = {job.dY, job.X, job.dW, job.lddy, job.ldx, job.lddw, 0};
+            for (int m = 0; m < job.N; m += 256)
+                for (int n = 0; n < job.K; n += 256)
+                    tile_table[tile++] = make_int4(j, m, n, 0);
+        }
+        check_hip(hipMemcpy(table, host.data(), host.size(), hipMemcpyHostToDevice), "wgrad list tables: ");
+    });
+}
+extern "C" int tgk_gemm_wgrad_list(hipStream_t stream, int M, int count, const TgkWgradJob *jobs, const void *table,
+                                   int accumulate, void *workspace, size_t workspace_bytes) {
+    return guarded([&] {
+        WgradListPlan plan;
+        std::string why;
+        if (!plan_wgrad_list(M, count, jobs, plan, why))
+            throw std::invalid_argument(why);
+        require(accumulate == 0, "gemm_wgrad_list: accumulate is not supported (every gradient is written once)");
+        require(table && !(reinterpret_cast<uintptr_t>(table) & 15), "gemm_wgrad_list: no table (see tgk_gemm_wgrad_list_prepare)");
+        require(plan.pieces_bytes == 0 ||
+                    (workspace && workspace_bytes >= plan.pieces_bytes && !(reinterpret_cast<uintptr_t>(workspace) & 15)),
+                "gemm_wgrad_list: workspace too small (see tgk_gemm_wgrad_list_workspace)");
+        WgradList w{};
+        w.jobs = static_cast<const WgradListJob *>(table);
+        w.tiles = reinterpret_cast<const int4 *>(static_cast<const unsigned char *>(table) + plan.jobs_bytes);
+        w.rounds = plan.rounds, w.rem_tiles = plan.rem_tiles, w.rem_splits = plan.rem_splits;
+        w.k_quads = M / 128;
+        w.accumulate = accumulate;
+        w.pieces = static_cast<float *>(workspace);
+        auto kernel = wgrad_list_kernel<256>;
+        constexpr size_t lds = 4 * (256 + 256) * 64;
+        static std::atomic<bool> configured[MAX_DEVICES];
+        const int device = current_device();
+        if (!configured[device].load(std::memory_order_acquire)) {
+            check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)),
+                      "gemm LDS size: ");
+            configured[device].store(true, std::memory_order_release);
+        }
+        const int blocks = plan.rounds ? plan.blocks : plan.rem_tiles * plan.rem_splits;
+        hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, w);
+        check_hip(hipGetLastError(), "wgrad list launch: ");
+        if (plan.rem_splits > 1) {
+            hipLaunchKernelGGL((wgrad_list_fold_kernel<256>), dim3(plan.rem_tiles * 8), dim3(256), 0, stream, w,
+                               plan.rounds * plan.blocks);
+            check_hip(hipGetLastError(), "wgrad list fold launch: ");
+        }
     });
 }
