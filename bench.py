@@ -2,7 +2,10 @@
 """Headline benchmark: training tokens/sec of the byte-level GPT d768 L12 H12 T1024 B16
 (the fourth benchmark configuration, configs[3]) on one MI355X, through the tg_* C ABI.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--kernels]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--kernels] [--config 3|4]
+
+--config 4 runs the long-context configuration (configs[4]: d1024 L24 H16 T4096 B4) through the same code and prints
+the same JSON shape; the default is the configuration the metric is quoted on.
 
 Prints ONE JSON line.  A step = sample a batch on the GPU, forward, backward, gradient norm, AdamW
 (nothing skipped; inputs are resident in HBM before the timed region).  After the timed region the
@@ -21,26 +24,37 @@ import time
 import numpy as np
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
-D, L, H, T, B, V = 768, 12, 12, 1024, 16, 256
+V = 256
+CONFIGS = {3: dict(D=768, L=12, H=12, T=1024, B=16), 4: dict(D=1024, L=24, H=16, T=4096, B=4)}
+D, L, H, T, B = (CONFIGS[3][k] for k in "DLHTB")
 F = 4 * D
 M = B * T
-# mean over the four projection shapes of 2 * (M*K + N*K + M*N) bytes: operands read and the result written once
-ALGORITHMIC_BYTES_PER_LAUNCH = sum(2 * (M * k + n * k + M * n) for n, k in
-                                   [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
 TRAFFIC_PROFILE = "profiles/gemm64_kc_kc_hbm_traffic.md"
 
 
+def select_config(index):
+    global D, L, H, T, B, F, M
+    D, L, H, T, B = (CONFIGS[index][k] for k in "DLHTB")
+    F, M = 4 * D, B * T
+
+
+def algorithmic_bytes_per_launch():
+    """Mean over the four projection shapes of 2 * (M*K + N*K + M*N) bytes: operands read and the result written once."""
+    return sum(2 * (M * k + n * k + M * n) for n, k in [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
+
+
 def hbm_traffic_per_launch():
-    """HBM bytes per launch of the dominant kernel, as the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary of
-    `--traffic-probe` states them ("... = 151.0 MB, against ..."): a figure of that profile, not of this run; None
-    when the file or the line is missing."""
+    """HBM bytes per launch of the dominant kernel and the kernel build they were measured on, as the committed
+    rocprofv3 FETCH_SIZE / WRITE_SIZE summary of `--traffic-probe` states them ("... = 151.0 MB, against ..." and a
+    "kernel source: ..." line): figures of that profile (configs[3] shapes), not of this run."""
     import re
-    try:
-        text = open(os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_PROFILE)).read()
-    except OSError:
-        return None
+    text = open(os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_PROFILE)).read()
     found = re.search(r"=\s*([0-9.]+)\s*MB,\s*against", text)
-    return float(found.group(1)) * 1e6 if found else None
+    source = re.search(r"kernel source:\s*(.+)", text)
+    if not found or not source:
+        sys.exit(f"bench.py: {TRAFFIC_PROFILE} no longer states the traffic per launch ('= X MB, against') or the "
+                 "kernel build it was measured on ('kernel source: ...')")
+    return float(found.group(1)) * 1e6, source.group(1).strip()
 
 
 def gemm_flops():
@@ -103,7 +117,7 @@ def zipf_bytes(n, rng, s=1.1):
 
 
 def cpu_baseline(sequences=8):
-    """The CPU checker on 8 of the step's 16 sequences (same model, B=8): forward, backward, AdamW."""
+    """The CPU checker on some of the step's sequences (same model, smaller batch): forward, backward, AdamW."""
     import oracle
     cfg = oracle.model(depth=L, context=T, batch=sequences, d_model=D, heads=H)
     w = oracle.init_weights(cfg)
@@ -136,7 +150,7 @@ def kernel_sweeps(out):
         torch.cuda.synchronize()
         return a.elapsed_time(b) / iters
 
-    for k, n in [(768, 2304), (768, 768), (768, 3072), (3072, 768)]:
+    for k, n in [(D, 3 * D), (D, D), (D, F), (F, D)]:
         x = torch.randn(M, k, device="cuda").bfloat16()
         w = torch.randn(n, k, device="cuda").bfloat16()
         dy = torch.randn(M, n, device="cuda").bfloat16()
@@ -183,12 +197,64 @@ def kernel_sweeps(out):
         keep.append((dy, x, dw))
         jobs[j] = WgradJob(n, k, dy.data_ptr(), n, x.data_ptr(), k, dw.data_ptr(), k)
     need = lib.tgk_gemm_wgrad_batch_workspace(M, 4, ctypes.addressof(jobs))
-    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
-    ms = timed(lambda: check(lib.tgk_gemm_wgrad_batch(stream, M, 4, ctypes.addressof(jobs), 0, ws.data_ptr(), need)))
-    flop = sum(2.0 * M * n * k for n, k in shapes)
-    print(json.dumps({"kernel": "gemm_wgrad_batch", "M": M, "shapes_N_K": shapes, "ms": round(ms, 4),
-                      "tflops": round(flop / ms / 1e9, 1),
-                      "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    if need:  # widths that are multiples of 192 only
+        ms = timed(lambda: check(lib.tgk_gemm_wgrad_batch(stream, M, 4, ctypes.addressof(jobs), 0, ws.data_ptr(), need)))
+        flop = sum(2.0 * M * n * k for n, k in shapes)
+        print(json.dumps({"kernel": "gemm_wgrad_batch", "M": M, "shapes_N_K": shapes, "ms": round(ms, 4),
+                          "tflops": round(flop / ms / 1e9, 1),
+                          "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}), file=out)
+    del keep, ws
+    # every weight gradient of the step in one launch, as the engine runs them (each layer with operands of its own)
+    shapes = [(D, F), (F, D), (D, D), (3 * D, D)] * L + [(V, D)]
+    keep, jobs = [], (WgradJob * len(shapes))()
+    for j, (n, k) in enumerate(shapes):
+        dy = torch.randn(M, n, device="cuda").bfloat16()
+        x = torch.randn(M, k, device="cuda").bfloat16()
+        dw = torch.empty(n, k, device="cuda")
+        keep.append((dy, x, dw))
+        jobs[j] = WgradJob(n, k, dy.data_ptr(), n, x.data_ptr(), k, dw.data_ptr(), k)
+    table_bytes = lib.tgk_gemm_wgrad_list_table_bytes(M, len(shapes), ctypes.addressof(jobs))
+    if table_bytes:
+        table = torch.empty(table_bytes, dtype=torch.uint8, device="cuda")
+        need = lib.tgk_gemm_wgrad_list_workspace(M, len(shapes), ctypes.addressof(jobs))
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        check(lib.tgk_gemm_wgrad_list_prepare(M, len(shapes), ctypes.addressof(jobs), table.data_ptr(), table_bytes))
+        ms = timed(lambda: check(lib.tgk_gemm_wgrad_list(stream, M, len(shapes), ctypes.addressof(jobs), table.data_ptr(),
+                                                         0, ws.data_ptr(), need)), iters=5)
+        flop = sum(2.0 * M * n * k for n, k in shapes)
+        print(json.dumps({"kernel": "gemm_wgrad_list", "M": M, "jobs": len(shapes), "ms": round(ms, 4),
+                          "tflops": round(flop / ms / 1e9, 1),
+                          "frac_of_bf16_peak": round(flop / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                          "operands": "N(0,1), cold (4.8 GB at configs[3])"}), file=out)
+        del table, ws
+    # comparators with a long reduction, the vendor library beside this library's kernel for the same layout:
+    # 8192^3 with both operands strided along the reduction (the weight-gradient layout), and one weight gradient of
+    # the step's largest shape both ways round
+    for rows, cols, reduced in [(8192, 8192, 8192), (F, D, M), (D, F, M)]:
+        a = torch.randn(reduced, rows, device="cuda").bfloat16()
+        b = torch.randn(reduced, cols, device="cuda").bfloat16()
+        c = torch.empty(rows, cols, device="cuda")
+        one = (WgradJob * 1)(WgradJob(rows, cols, a.data_ptr(), rows, b.data_ptr(), cols, c.data_ptr(), cols))
+        table_bytes = lib.tgk_gemm_wgrad_list_table_bytes(reduced, 1, ctypes.addressof(one))
+        table = torch.empty(max(table_bytes, 16), dtype=torch.uint8, device="cuda")
+        need = lib.tgk_gemm_wgrad_list_workspace(reduced, 1, ctypes.addressof(one))
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        flop = 2.0 * rows * cols * reduced
+        line = {"kernel": "long_reduction", "C": [rows, cols], "reduced": reduced, "layout": "A^T B, both [reduced][n]"}
+        if table_bytes:
+            check(lib.tgk_gemm_wgrad_list_prepare(reduced, 1, ctypes.addressof(one), table.data_ptr(), table_bytes))
+            ms = timed(lambda: check(lib.tgk_gemm_wgrad_list(stream, reduced, 1, ctypes.addressof(one), table.data_ptr(), 0,
+                                                             ws.data_ptr(), need)), iters=10)
+            line["tflops"] = round(flop / ms / 1e9, 1)
+        ms = timed(lambda: torch.matmul(a.t(), b), iters=10)
+        line["vendor_library_tflops"] = round(flop / ms / 1e9, 1)
+        if rows == cols:  # the library's best layout for the same product, for scale
+            ms = timed(lambda: torch.matmul(a, b.t()), iters=10)
+            line["vendor_library_tflops_both_contiguous"] = round(flop / ms / 1e9, 1)
+        print(json.dumps(line), file=out)
+        del a, b, c, table, ws
+    del keep
     d = H * 64
     qkv = torch.randn(M, 3 * d, device="cuda").bfloat16()
     do = torch.randn(M, d, device="cuda").bfloat16()
@@ -253,7 +319,10 @@ def main():
     ap.add_argument("--kernels", action="store_true", help="also print the isolated kernel sweeps to stderr")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="run only the copy + forward GEMM dispatches used to read HBM traffic counters")
+    ap.add_argument("--config", type=int, default=3, choices=sorted(CONFIGS),
+                    help="3: d768 L12 T1024 B16 (the metric's configuration); 4: d1024 L24 T4096 B4")
     args = ap.parse_args()
+    select_config(args.config)
     if args.traffic_probe:
         return traffic_probe()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -294,6 +363,8 @@ def main():
         rate = amount / (per_step_ms * 1e-3) / 1e12 if per_step_ms > 0 else 0.0
         classes[name] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // 3,
                          ("tflops" if kind == "flop" else "tb_per_s"): round(rate, 2)}
+    traffic, traffic_source = hbm_traffic_per_launch() if args.config == 3 else (None, "not measured for this configuration")
+    tile = "128,192" if D % 192 == 0 else "128,192 and 128,128"
     # dominant MFMA kernel: gemm64_kernel<128,192,true,true,EpilogueBf16As<mode>> - both operands contiguous along
     # the reduced dimension, one instantiation per epilogue (plain, + residual, GELU, GELU') - which runs the forward
     # block projections (on the weights) and the dgrads (on their transposed copies): 8 launches per layer, 96 per
@@ -305,7 +376,7 @@ def main():
     achieved = flops_per_launch / (launch_ms * 1e-3) / 1e12
     ms_per_step = seconds / args.steps * 1e3
     result = {
-        "metric": "train tokens/sec at d768 L12 T1024 (1 GPU)",
+        "metric": f"train tokens/sec at d{D} L{L} T{T} (1 GPU)",
         "value": round(args.steps * M / seconds, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -317,29 +388,30 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "configs[3]: full training step, byte-level GPT d_model=768 L=12 H=12 T=1024 B=16 "
-                               "ffn=3072 vocab=256, bf16 weights with fp32 masters, AdamW lr 3e-4 betas 0.9/0.95 "
-                               "wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
+        "config": {"workload": f"configs[{args.config}]: full training step, byte-level GPT d_model={D} L={L} H={H} "
+                               f"T={T} B={B} ffn={F} vocab=256, bf16 weights with fp32 masters, AdamW lr 3e-4 betas "
+                               "0.9/0.95 wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
                    "global_batch": B, "seq_len": T, "parameters": params, "parallelism": "single GPU"},
         "roofline": {"bound": "mfma",
-                     "kernel": "gemm64_kernel<128,192,true,true,EpilogueBf16As<mode>>, its four epilogue "
+                     "kernel": f"gemm64_kernel<{tile},true,true,EpilogueBf16As<mode>>, its four epilogue "
                                "instantiations together (forward block projections and dgrads: QKV, attention-out, "
                                "MLP-up, MLP-down)",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": hbm_traffic_per_launch(),
+                     "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                      "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE of --traffic-probe, "
                                      "calibrated on a copy of known size)",
-                     "traffic_source": TRAFFIC_PROFILE + " (read from that committed profile, not measured in this run)",
-                     "algorithmic_bytes_per_launch": ALGORITHMIC_BYTES_PER_LAUNCH,
+                     "traffic_source": (TRAFFIC_PROFILE + " (read from that committed profile, not measured in this "
+                                        "run; taken on: " + traffic_source + ")") if traffic else traffic_source,
+                     "algorithmic_bytes_per_launch": algorithmic_bytes_per_launch(),
                      "flops_per_launch": flops_per_launch, "avg_launch_ms": round(launch_ms, 5)},
         "classes": classes,
-        # 9.45 TFLOP of algorithmic work per step (attention causal-counted, backward = 2.5 x forward)
+        # algorithmic work per step (9.45 TFLOP at configs[3]; attention causal-counted, backward = 2.5 x forward)
         "model_tflops": round((3 * L * sum(gemm_flops()) + 3 * 2.0 * M * V * D +
                                L * 3.5 * 4.0 * B * H * T * T * 64 / 2) / (ms_per_step * 1e-3) / 1e12, 1),
         "loss_first_last": [round(float(losses[0]), 4), round(float(losses[-1]), 4)],
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline()
+        result["cpu_baseline"] = cpu_baseline(8 if args.config == 3 else 1)
     if args.kernels:
         kernel_sweeps(sys.stderr)
     print(json.dumps(result))
