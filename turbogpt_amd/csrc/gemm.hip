@@ -737,6 +737,218 @@ __global__ __launch_bounds__(256, 2) void gemm64_kernel(const bf16_t *__restrict
     wait_vmcnt<0>();
 }
 
+TG_DEVICE uint32_t kc64_frag16_offset(int row0, int ks, int lane) { // TileKC64::frag16's address
+    const int row = row0 + (lane & 15), chunk = (ks * 4 + (lane >> 4)) ^ ((row >> 1) & 7);
+    return uint32_t(row * 128 + chunk * 16);
+}
+// ---- 256 x 192 tiles, one wave per SIMD: forward and input-gradient products with a long or plain epilogue ------
+// C = A B^T with both operands k-contiguous, a 256 x 192 tile per block, four waves of 128 x 96 outputs each, one
+// block per compute unit.  What bounds these products is a compute unit's copy path: bytes per flop, whole
+// cache lines per request, and how many requests it keeps in flight.  Hence: 9.1 bytes per kFLOP without relying on
+// another block's lines in L1; 64 k per stage (every request a whole 128-byte line); and rings of different depth for
+// the two operands - three slots for A (activations, streamed from beyond the L2: a copy has two stages to land) and
+// two for B (the weights, mostly L2 hits: one stage), 144 KB of LDS.  With a lone wave per SIMD the fragments of the
+// next 32-k step are read into a second register set between the matrix instructions of the current one:
+//   first half of stage g : matrix instructions on (g, k 0..31), fragment reads of (g, k 32..63)
+//   wait (all but A's youngest stage), barrier: stage g + 1 is visible, nobody reads stage g's slots any more
+//   second half           : matrix instructions on (g, k 32..63), copies of B's stage g + 2 and A's stage g + 3,
+//                           fragment reads of (g + 1, k 0..31)
+// The loop is unrolled over six stages (the rings' common period): the reduced dimension is a multiple of 384.
+template <class Epilogue>
+__global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restrict__ A, int lda,
+                                                       const bf16_t *__restrict__ B, int ldb, int k_sixes,
+                                                       int tiles_n, int tiles_total, int xcd_cols,
+                                                       Epilogue epilogue) {
+    constexpr int BM = 256, BN = 192;
+    constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32, AF = 2 * FM, BF = 2 * FN, MFMAS = AF * BF;
+    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, B_RING = 3 * A_BYTES, BUFFERS = B_RING + 2 * B_BYTES;
+    constexpr int LA = BM * 128 / 4096, LB = BN * 128 / 4096, LOADS = LA + LB; // copies per wave and stage
+    constexpr int READ_EVERY = MFMAS / (AF + BF), COPY_EVERY = MFMAS / LOADS;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t smem_base = lds_address(smem);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    const int stride = gridDim.x;
+
+    auto locate = [&](int item, int &m0, int &n0) {
+        int tile_m, tile_n;
+        if ((tiles_total & 7) == 0 && xcd_cols > 1) {
+            const int xcd = item & 7, index = item >> 3;
+            const int cols = tiles_n / xcd_cols, rows = (tiles_total / tiles_n) / (8 / xcd_cols);
+            tile_m = (xcd / xcd_cols) * rows + index / cols;
+            tile_n = (xcd % xcd_cols) * cols + index % cols;
+        } else {
+            const int logical = (tiles_total & 7) == 0 ? (item & 7) * (tiles_total >> 3) + (item >> 3) : item;
+            tile_m = logical / tiles_n;
+            tile_n = logical % tiles_n;
+        }
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
+    };
+
+    // ---- producers: A three stages ahead of the consumer, B two --------------------------------------------------
+    const int copy_row = lane >> 3, copy_chunk = (lane & 7) ^ ((((wave & 1) * 4) + (lane >> 4)) & 7);
+    const uint32_t la = uint32_t(copy_row * lda + copy_chunk * 8) * 2, lb = uint32_t(copy_row * ldb + copy_chunk * 8) * 2;
+    const int64_t a_rows32 = int64_t(32) * lda * 2, b_rows32 = int64_t(32) * ldb * 2;
+    // wave-uniform: the stage either producer copies next (this wave's first row of it), the first stage of the tile
+    // after the current one, and the bytes from one stage to the next (0 once the list is exhausted: the copies go
+    // on, re-reading a stage into slots nobody consumes, and the loop stays straight-line code)
+    const char *pa_at = nullptr, *pb_at = nullptr, *a_next = nullptr, *b_next = nullptr;
+    int64_t pa_step = 128, pb_step = 128, next_step = 128;
+    auto tile_origin = [&](int item, const char *&a, const char *&b) {
+        int m0, n0;
+        locate(item, m0, n0);
+        a = reinterpret_cast<const char *>(A + int64_t(m0 + wave * 8) * lda);
+        b = reinterpret_cast<const char *>(B + int64_t(n0 + wave * 8) * ldb);
+    };
+    auto prepare_next = [&](int item) { // keeps the current origins when there is no further tile
+        if (item < tiles_total)
+            tile_origin(item, a_next, b_next);
+        else
+            next_step = 0;
+    };
+    auto copy_a = [&](int n, int slot) __attribute__((always_inline)) {
+        async_copy16(smem_base + uint32_t(slot * A_BYTES + (n * 4 + wave) * 1024), pa_at + n * a_rows32, la);
+    };
+    auto copy_b = [&](int n, int slot) __attribute__((always_inline)) {
+        async_copy16(smem_base + uint32_t(B_RING + slot * B_BYTES + (n * 4 + wave) * 1024), pb_at + n * b_rows32, lb);
+    };
+    if (int(blockIdx.x) >= tiles_total)
+        return;
+    tile_origin(blockIdx.x, pa_at, pb_at);
+    a_next = pa_at, b_next = pb_at;
+    prepare_next(blockIdx.x + stride);
+    // stages 0 and 1 of both, then A's stage 2 (so that A's youngest stage is the last one issued, as in the loop)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int n = 0; n < LB; ++n)
+            copy_b(n, s);
+#pragma unroll
+        for (int n = 0; n < LA; ++n)
+            copy_a(n, s);
+        pa_at += pa_step, pb_at += pb_step;
+    }
+#pragma unroll
+    for (int n = 0; n < LA; ++n)
+        copy_a(n, 2);
+    pa_at += pa_step;
+
+    // ---- consumer ----------------------------------------------------------------------------------------------------
+    uint32_t fa_at[2], fa_far[2], fb_at[2]; // fragment 0 of either 32-k step; fragment i lies 2048 i bytes further on
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        fa_at[ks] = kc64_frag16_offset(wm, ks, lane);
+        fa_far[ks] = fa_at[ks] + 2 * A_BYTES; // slot 2 lies beyond a ds_read's 16-bit offset
+        fb_at[ks] = B_RING + kc64_frag16_offset(wn, ks, lane);
+    }
+    auto read_fragment = [&](bf16x8 (&fa)[AF], bf16x8 (&fb)[BF], int slot_a, int slot_b, int ks, int f)
+                             __attribute__((always_inline)) {
+        if (f < AF)
+            fa[f] = slot_a == 2 ? *reinterpret_cast<const bf16x8 *>(smem + fa_far[ks] + f * 2048)
+                                : *reinterpret_cast<const bf16x8 *>(smem + fa_at[ks] + slot_a * A_BYTES + f * 2048);
+        else
+            fb[f - AF] = *reinterpret_cast<const bf16x8 *>(smem + fb_at[ks] + slot_b * B_BYTES + (f - AF) * 2048);
+    };
+    f32x4 acc[FM][FN][2][2];
+    bool last_six = k_sixes == 1; // the consumer is in a tile's last six stages
+    // One 32-k step on `cur`; meanwhile the fragments of (next slots, next_ks) are read into `next`, and, in a
+    // stage's second half, the copies go out: B first, A behind it (so that a wait can leave A's youngest stage out).
+    auto half = [&](auto copy_tag, int next_a_slot, int next_b_slot, int next_ks, int copy_a_slot, int copy_b_slot,
+                    const bf16x8 (&cur_a)[AF], const bf16x8 (&cur_b)[BF], bf16x8 (&next_a)[AF], bf16x8 (&next_b)[BF])
+                    __attribute__((always_inline)) {
+        constexpr bool COPY = decltype(copy_tag)::value;
+#pragma unroll
+        for (int j = 0; j < BF; ++j)
+#pragma unroll
+            for (int i = 0; i < AF; ++i) {
+                // accumulators pinned to the accumulation registers (see wgrad_list_kernel)
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                             : "+a"(acc[i >> 1][j >> 1][i & 1][j & 1])
+                             : "v"(cur_b[j]), "v"(cur_a[i]));
+                const int q = j * AF + i;
+                if (q % READ_EVERY == 0 && q / READ_EVERY < AF + BF)
+                    read_fragment(next_a, next_b, next_a_slot, next_b_slot, next_ks, q / READ_EVERY);
+                if (COPY && q % COPY_EVERY == 1 % COPY_EVERY && q / COPY_EVERY < LOADS) {
+                    const int n = q / COPY_EVERY;
+                    if (n < LB)
+                        copy_b(n, copy_b_slot);
+                    else
+                        copy_a(n - LB, copy_a_slot);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    };
+    // stage g = STAGE (mod 6): A slot g % 3, B slot g % 2
+    auto stage = [&](auto stage_tag, bf16x8 (&fa0)[AF], bf16x8 (&fb0)[BF], bf16x8 (&fa1)[AF], bf16x8 (&fb1)[BF])
+                     __attribute__((always_inline)) {
+        constexpr int G = decltype(stage_tag)::value, SA = G % 3, SB = G % 2;
+        // In a tile's last six stages the producers cross into the next tile: A with the copies of stage 3 (three
+        // stages ahead), B with those of stage 4.  Selects, not branches.
+        if (G == 3 && last_six)
+            pa_at = a_next, pa_step = next_step;
+        if (G == 4 && last_six)
+            pb_at = b_next, pb_step = next_step;
+        half(std::false_type{}, SA, SB, 1, 0, 0, fa0, fb0, fa1, fb1);
+        wait_vmcnt<LA>();                   // everything but A's youngest stage has landed
+        __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): and this wave's reads of this stage are done
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        // copies: B's stage g + 2 into B slot g % 2, A's stage g + 3 into A slot g % 3 (the slots this stage leaves)
+        half(std::true_type{}, (SA + 1) % 3, SB ^ 1, 0, SA, SB, fa1, fb1, fa0, fb0);
+        pa_at += pa_step, pb_at += pb_step;
+    };
+    const bf16x8 zeros = {0, 0, 0, 0, 0, 0, 0, 0};
+    auto clear = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    asm volatile("s_nop 4\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %1, 0"
+                                 : "+a"(acc[i][j][t >> 1][t & 1])
+                                 : "v"(zeros)); // zeroed in place, wait states included (see wgrad_list_kernel)
+    };
+    bf16x8 fa0[AF], fb0[BF], fa1[AF], fb1[BF];
+    wait_vmcnt<LA + LOADS>(); // stage 0
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int f = 0; f < AF + BF; ++f)
+        read_fragment(fa0, fb0, 0, 0, 0, f);
+    unsigned char *mine = smem + BUFFERS + wave * 2048;
+    int item = blockIdx.x, sixes_left = k_sixes;
+    clear();
+    for (;;) {
+        stage(std::integral_constant<int, 0>{}, fa0, fb0, fa1, fb1);
+        stage(std::integral_constant<int, 1>{}, fa0, fb0, fa1, fb1);
+        stage(std::integral_constant<int, 2>{}, fa0, fb0, fa1, fb1);
+        stage(std::integral_constant<int, 3>{}, fa0, fb0, fa1, fb1);
+        stage(std::integral_constant<int, 4>{}, fa0, fb0, fa1, fb1);
+        stage(std::integral_constant<int, 5>{}, fa0, fb0, fa1, fb1);
+        if (--sixes_left) {
+            last_six = sixes_left == 1;
+            continue;
+        }
+        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7"); // the compiler does not know that matrix instructions wrote the accumulators
+        int m0, n0;
+        locate(item, m0, n0);
+        u32x4 aux[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}};
+        if (epilogue.wants_aux())
+            load_aux_pair<FM, FN>(epilogue, 0, m0 + wm, n0 + wn, lane, aux);
+        staged_store_bf16<FM, FN>(acc, aux, mine, epilogue, m0 + wm, n0 + wn, lane);
+        wait_vmcnt<0>(); // loads and stores drained: the counter holds nothing but copies again
+        item += stride;
+        if (item >= tiles_total)
+            break;
+        prepare_next(item + stride);
+        sixes_left = k_sixes;
+        last_six = k_sixes == 1;
+        clear();
+    }
+    wait_vmcnt<0>();
+}
+
 // ---- several weight gradients in one launch ------------------------------------------------------
 // dW_j[N_j][K_j] = dY_j^T X_j for up to four (dY, X) pairs that share the reduced dimension (the tokens).  One
 // matrix rarely has as many 128x192 tiles as the GPU holds blocks, and split into as many token ranges as fill
@@ -1362,6 +1574,43 @@ void launch_gemm64(hipStream_t stream, Tile tile, const bf16_t *A, int lda, cons
         launch_gemm64_tile<128, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
 }
 
+// The 256 x 192 kernel takes products with a plain or residual epilogue whose tiles fill the compute units a whole
+// number of times (or nearly): one block per unit, nothing to cover a tail or a long epilogue (the GELU epilogues
+// stay with gemm64_kernel, where the second block of a unit multiplies meanwhile).
+bool takes_256x192(int M, int N, int K, int mode) {
+    if (M % 256 || N % 192 || K % 384 || (mode != EPI_PLAIN && mode != EPI_RESIDUAL))
+        return false;
+    const int tiles = (M / 256) * (N / 192), units = compute_units();
+    const int rounds = (tiles + units - 1) / units;
+    return tiles * 10 >= rounds * units * 9; // at least 90 % of the last round filled
+}
+template <class Epilogue>
+void launch_gemm256(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
+                    const Epilogue &epilogue) {
+    auto kernel = gemm256_kernel<Epilogue>;
+    constexpr size_t lds = 3 * 256 * 128 + 2 * 192 * 128 + 4 * 2048;
+    static std::atomic<bool> configured[MAX_DEVICES];
+    const int device = current_device();
+    if (!configured[device].load(std::memory_order_acquire)) {
+        check_hip(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)),
+                  "gemm LDS size: ");
+        configured[device].store(true, std::memory_order_release);
+    }
+    const int tiles_m = M / 256, tiles_n = N / 192, tiles = tiles_m * tiles_n;
+    const int units = compute_units(), blocks = tiles < units ? tiles : units;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, A, lda, B, ldb, K / 384, tiles_n, tiles,
+                       xcd_columns(tiles_m, tiles_n, 256, 192, K, blocks), epilogue);
+    check_hip(hipGetLastError(), "gemm launch: ");
+}
+void launch_gemm256_bf16(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
+                         const EpilogueBf16 &e) {
+    if (e.mode == EPI_RESIDUAL)
+        launch_gemm256(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_RESIDUAL>{e});
+    else
+        launch_gemm256(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_PLAIN>{e});
+}
+
 // bf16 epilogues of the 64-k kernel: one instantiation per mode
 template <bool AKC, bool BKC>
 void launch_gemm64_bf16(hipStream_t stream, Tile tile, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N,
@@ -1415,7 +1664,9 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
             check_operand(gelu_out, ldg, "gelu_out");
             e.out2 = gelu_out, e.ld_out2 = ldg, e.mode = EPI_GELU;
         }
-        if (takes_64(tile, K))
+        if (takes_256x192(M, N, K, e.mode))
+            launch_gemm256_bf16(stream, X, ldx, W, ldw, M, N, K, e);
+        else if (takes_64(tile, K))
             launch_gemm64_bf16<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, e);
         else
             dispatch_gemm<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, 1, e);
@@ -1485,7 +1736,9 @@ extern "C" int tgk_gemm_dgrad_t(hipStream_t stream, int M, int N, int K, const u
             e.aux = gelu_pre, e.ld_aux = ldu, e.mode = EPI_GELU_BWD;
         }
         // C[m][i] = sum_o dY[m][o] Wt[i][o]: the forward product with (rows, reduced) = (K, N)
-        if (takes_64(tile, N))
+        if (takes_256x192(M, K, N, e.mode))
+            launch_gemm256_bf16(stream, dY, lddy, Wt, ldwt, M, K, N, e);
+        else if (takes_64(tile, N))
             launch_gemm64_bf16<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, e);
         else
             dispatch_gemm<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, 1, e);
