@@ -98,6 +98,9 @@ struct EpilogueBf16 {
 // code the stores of a block stay in flight while the next is rounded and transposed.
 template <int MODE> struct EpilogueBf16As {
     static constexpr bool BF16 = true;
+    // vector-memory instructions per 32 x 32 block of the staged epilogue: two 16-byte stores (four with the GELU
+    // output), two 16-byte loads of the second input
+    static constexpr int MEMORY_OPS_PER_BLOCK = MODE == EPI_PLAIN ? 2 : 4;
     EpilogueBf16 any;
     TG_DEVICE bool wants_aux() const { return MODE == EPI_RESIDUAL || MODE == EPI_GELU_BWD; }
     TG_DEVICE u32x4 load_aux(int m, int n) const { return any.load_aux(m, n); }
@@ -852,6 +855,8 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
     };
     f32x4 acc[FM][FN][2][2];
     bool last_six = k_sixes == 1; // the consumer is in a tile's last six stages
+    bool behind_epilogue = false;
+    static_assert(LA + FM * FN * Epilogue::MEMORY_OPS_PER_BLOCK < 64, "the wait count has six bits");
     // One 32-k step on `cur`; meanwhile the fragments of (next slots, next_ks) are read into `next`, and, in a
     // stage's second half, the copies go out: B first, A behind it (so that a wait can leave A's youngest stage out).
     auto half = [&](auto copy_tag, int next_a_slot, int next_b_slot, int next_ks, int copy_a_slot, int copy_b_slot,
@@ -890,7 +895,14 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
         if (G == 4 && last_six)
             pb_at = b_next, pb_step = next_step;
         half(std::false_type{}, SA, SB, 1, 0, 0, fa0, fb0, fa1, fb1);
-        wait_vmcnt<LA>();                   // everything but A's youngest stage has landed
+        // Everything but A's youngest stage has landed.  A wave's loads and stores retire in order through one counter;
+        // behind a tile's epilogue its loads and stores are the youngest operations, and their number is known.
+        if (G == 0 && behind_epilogue)
+            wait_vmcnt<LA + FM * FN * Epilogue::MEMORY_OPS_PER_BLOCK>();
+        else
+            wait_vmcnt<LA>();
+        if (G == 0)
+            behind_epilogue = false;
         __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): and this wave's reads of this stage are done
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -937,7 +949,7 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
         if (epilogue.wants_aux())
             load_aux_pair<FM, FN>(epilogue, 0, m0 + wm, n0 + wn, lane, aux);
         staged_store_bf16<FM, FN>(acc, aux, mine, epilogue, m0 + wm, n0 + wn, lane);
-        wait_vmcnt<0>(); // loads and stores drained: the counter holds nothing but copies again
+        behind_epilogue = true; // the stores stay in flight under the next tile's first stage
         item += stride;
         if (item >= tiles_total)
             break;
@@ -1224,16 +1236,9 @@ __global__ __launch_bounds__(256, 1) void wgrad_list_kernel(const WgradList w) {
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32, AF = 2 * FM, BF = 2 * FN, MFMAS = AF * BF;
     constexpr int LA = TA::LOADS, LB = TB::LOADS, LOADS = LA + LB;
     constexpr int A_RING = S * TA::BYTES;
-#ifndef WL_READ_EVERY
-#define WL_READ_EVERY 3
-#endif
-#ifndef WL_COPY_EVERY
-#define WL_COPY_EVERY (MFMAS / LOADS)
-#endif
-#ifndef WL_COPY_FIRST
-#define WL_COPY_FIRST 1
-#endif
-    constexpr int READ_EVERY = WL_READ_EVERY, COPY_EVERY = WL_COPY_EVERY, COPY_FIRST = WL_COPY_FIRST;
+    // a fragment read behind every third matrix instruction, a copy behind every eighth (measured: the best of five
+    // placements, by 4 %)
+    constexpr int READ_EVERY = 3, COPY_EVERY = MFMAS / LOADS, COPY_FIRST = 1;
     extern __shared__ __align__(16) unsigned char smem[];
     const uint32_t smem_base = lds_address(smem);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1326,14 +1331,10 @@ __global__ __launch_bounds__(256, 1) void wgrad_list_kernel(const WgradList w) {
                              : "+a"(acc[i >> 1][j >> 1][i & 1][j & 1])
                              : "v"(cur_b[j]), "v"(cur_a[i]));
                 const int q = j * AF + i;
-#ifndef WL_NO_READ
                 if (q % READ_EVERY == 0 && q / READ_EVERY < AF + BF)
                     read_fragment(next_a, next_b, NEXT, q / READ_EVERY);
-#endif
-#ifndef WL_NO_COPY
                 if (q >= COPY_FIRST && (q - COPY_FIRST) % COPY_EVERY == 0 && (q - COPY_FIRST) / COPY_EVERY < LOADS)
                     copy_one((q - COPY_FIRST) / COPY_EVERY, SLOT);
-#endif
                 __builtin_amdgcn_sched_barrier(0);
             }
         p_a += a_step, p_b += b_step;
