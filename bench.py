@@ -39,8 +39,10 @@ def select_config(index):
 
 
 def algorithmic_bytes_per_launch():
-    """Mean over the four projection shapes of 2 * (M*K + N*K + M*N) bytes: operands read and the result written once."""
-    return sum(2 * (M * k + n * k + M * n) for n, k in [(3 * D, D), (D, D), (F, D), (D, F)]) / 4
+    """Mean over the dominant kernel's six launches per layer of 2 * (M*K + N*K + M*N [+ M*N residual]) bytes: operands
+    read once, the result written once."""
+    launches = [(3 * D, D, 0), (D, D, 1), (D, F, 1), (D, F, 0), (D, D, 0), (D, 3 * D, 0)]  # (N, K, residual read)
+    return sum(2 * (M * k + n * k + M * n * (1 + r)) for n, k, r in launches) / len(launches)
 
 
 def hbm_traffic_per_launch():
@@ -69,9 +71,12 @@ def class_work():
     attn_fwd = 4.0 * B * H * T * T * 64 / 2  # causal-counted
     act, wide = M * D * 2, M * F * 2
     params = V * D * 2 + T * D + L * (4 * D + 4 * D * D + 2 * F * D) + 2 * D
+    qkv, out, up, down = gemm_flops()
     return {
-        "gemm_fwd": ("flop", L * per_layer),
-        "gemm_dgrad": ("flop", L * per_layer),
+        "gemm_fwd": ("flop", L * (qkv + out + down)),     # plain / residual epilogues
+        "gemm_fwd_gelu": ("flop", L * up),                # MLP-up: pre-activation and GELU written
+        "gemm_dgrad": ("flop", L * (qkv + out + up)),     # plain epilogue
+        "gemm_dgrad_gelu": ("flop", L * down),            # MLP-down dgrad times GELU'
         "gemm_wgrad": ("flop", L * per_layer),
         "attn_fwd": ("flop", L * attn_fwd),
         "attn_bwd": ("flop", L * attn_fwd * 2.5),
@@ -364,16 +369,18 @@ def main():
         classes[name] = {"ms_per_step": round(per_step_ms, 4), "launches_per_step": launches // 3,
                          ("tflops" if kind == "flop" else "tb_per_s"): round(rate, 2)}
     traffic, traffic_source = hbm_traffic_per_launch() if args.config == 3 else (None, "not measured for this configuration")
-    tile = "128,192" if D % 192 == 0 else "128,192 and 128,128"
-    # dominant MFMA kernel: gemm64_kernel<128,192,true,true,EpilogueBf16As<mode>> - both operands contiguous along
-    # the reduced dimension, one instantiation per epilogue (plain, + residual, GELU, GELU') - which runs the forward
-    # block projections (on the weights) and the dgrads (on their transposed copies): 8 launches per layer, 96 per
-    # step, the same four shapes in both directions.
+    # Dominant MFMA kernel: the forward block projections and input gradients with a plain or residual epilogue, six
+    # launches per layer - QKV, attention-out and MLP-down forward (on the weights), MLP-up, attention-out and QKV dgrad
+    # (on the transposed copies).  Widths that 192 and 384 divide run them on gemm256_kernel<EpilogueBf16As<0|1>>
+    # (256 x 192 tiles), others on gemm64_kernel<128,128|192,true,true,EpilogueBf16As<0|1>>.
     fwd_ms, fwd_launches = profile["gemm_fwd"]
     dgrad_ms, dgrad_launches = profile["gemm_dgrad"]
     launch_ms = (fwd_ms + dgrad_ms) / (fwd_launches + dgrad_launches)
-    flops_per_launch = sum(gemm_flops()) / 4
+    qkv, out, up, down = gemm_flops()
+    flops_per_launch = (2 * qkv + 2 * out + up + down) / 6
     achieved = flops_per_launch / (launch_ms * 1e-3) / 1e12
+    kernel = ("gemm256_kernel<EpilogueBf16As<0|1>> (256x192 tiles, one wave per SIMD)" if D % 384 == 0 else
+              "gemm64_kernel<128,128|192,true,true,EpilogueBf16As<0|1>>")
     ms_per_step = seconds / args.steps * 1e3
     result = {
         "metric": f"train tokens/sec at d{D} L{L} T{T} (1 GPU)",
@@ -393,9 +400,8 @@ def main():
                                "0.9/0.95 wd 0.1 clip 1.0, Zipf(1.1) bytes sampled on the GPU",
                    "global_batch": B, "seq_len": T, "parameters": params, "parallelism": "single GPU"},
         "roofline": {"bound": "mfma",
-                     "kernel": f"gemm64_kernel<{tile},true,true,EpilogueBf16As<mode>>, its four epilogue "
-                               "instantiations together (forward block projections and dgrads: QKV, attention-out, "
-                               "MLP-up, MLP-down)",
+                     "kernel": kernel + ", plain and residual epilogues together: QKV, attention-out, MLP-down "
+                               "forward and MLP-up, attention-out, QKV dgrad (six launches per layer)",
                      "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                      "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE of --traffic-probe, "

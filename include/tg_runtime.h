@@ -92,9 +92,9 @@ TG_API int tg_synchronize(Engine *engine);
  * with a HIP event pair around every operator launch on the engine's stream, and returns summed
  * milliseconds and launch counts per operator class.  Synchronises. */
 enum {
-    TG_CLASS_GEMM_FWD = 0,   /* block projections forward (QKV, attention-out, MLP-up, MLP-down) */
-    TG_CLASS_GEMM_DGRAD = 1, /* their input gradients */
-    TG_CLASS_GEMM_WGRAD = 2, /* their weight gradients, split-K reduction included */
+    TG_CLASS_GEMM_FWD = 0,   /* block projections forward with a plain or residual epilogue (QKV, attention-out, MLP-down) */
+    TG_CLASS_GEMM_DGRAD = 1, /* input gradients with a plain epilogue (MLP-up, attention-out, QKV) */
+    TG_CLASS_GEMM_WGRAD = 2, /* the weight gradients, partial-sum folds included */
     TG_CLASS_ATTN_FWD = 3,
     TG_CLASS_ATTN_BWD = 4,
     TG_CLASS_LAYERNORM_FWD = 5,
@@ -102,7 +102,9 @@ enum {
     TG_CLASS_HEAD = 7,       /* vocabulary projection: forward, dgrad, wgrad */
     TG_CLASS_OTHER = 8,      /* sampling, embedding, cross-entropy, loss means */
     TG_CLASS_OPTIMIZER = 9,  /* gradient norm + AdamW */
-    TG_CLASSES = 10
+    TG_CLASS_GEMM_FWD_GELU = 10,   /* MLP-up forward: two outputs, pre-activation and GELU */
+    TG_CLASS_GEMM_DGRAD_GELU = 11, /* MLP-down input gradient times GELU' of the saved pre-activation */
+    TG_CLASSES = 12
 };
 TG_API int tg_profile_step(Engine *engine, float *class_ms, int *class_launches, int classes);
 

@@ -134,7 +134,10 @@ TGK_API size_t tgk_attn_bwd_workspace(int B, int H, int T);
  * 8 MiB per GPU the library runs on, held until the process ends.  B*H*T <= tgk_attn_bwd_static_max_rows()
  * (1048576); larger shapes are rejected and need tgk_attn_bwd.  The call allocates and frees nothing.  All
  * calls on one GPU share the array: calls that overlap on one GPU (different streams or threads) race.
- * Same kernels and results, bit for bit, as tgk_attn_bwd. */
+ * Same kernels and results, bit for bit, as tgk_attn_bwd.  The array's address is looked up once per device, on the
+ * first tgk_attn_bwd_static or tgk_attn_bwd_static_max_rows call made with that device current: make one of them
+ * outside any stream capture on every device that will run it (a lookup inside a capture may be refused), and call
+ * with the stream's device current - the array used is the current device's. */
 TGK_API int tgk_attn_bwd_static(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
                                 const uint16_t *K, const uint16_t *V, int ld, const uint16_t *O, int ldo,
                                 const float *lse, const uint16_t *dO, int lddo, uint16_t *dQ, uint16_t *dK,

@@ -131,6 +131,32 @@ def test_full_size_config3_properties(orc):
     assert (o.view(B, T, H, 64).float().abs().amax(1) <= v.abs().amax(1) * 1.01).all()
 
 
+def test_long_context_config4_shape_against_the_checker(orc):
+    """B4 H16 T4096 hd64 (the attention of BASELINE configs[4]): one (batch, head) pair in full against the checker
+    (the T = 4096 key loop, 64 key tiles per query tile), the whole tensor held to the size-independent properties."""
+    rng = np.random.default_rng(44)
+    B, H, T = 4, 16, 4096
+    d = H * 64
+    qkv = torch.from_numpy(rng.standard_normal((B * T, 3 * d), dtype=np.float32)).bfloat16().cuda()
+    do = torch.from_numpy(rng.standard_normal((B * T, d), dtype=np.float32)).bfloat16().cuda()
+    o, lse = run_fwd(qkv, B, H, T, 0.125)
+    dqkv = run_bwd(qkv, o, lse, do, B, H, T, 0.125)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(dqkv.float()).all()
+    b, h = 2, 9
+    cols = np.r_[h * 64:(h + 1) * 64]
+    sub = host(qkv.view(B, T, 3 * d)[b])[:, np.r_[cols, d + cols, 2 * d + cols]]
+    want_o, want_lse = orc.attn_fwd(sub, 1, 1, T, 64, 0.125)
+    assert rel(host(o.view(B, T, d)[b])[:, cols], want_o) < 1e-2
+    np.testing.assert_allclose(host(lse[b, h]), want_lse[0, 0], atol=2e-3, rtol=1e-4)
+    want_d = orc.attn_bwd(sub, want_o, want_lse, host(do.view(B, T, d)[b])[:, cols], 1, 1, T, 64, 0.125)
+    got_d = host(dqkv.view(B, T, 3 * d)[b])[:, np.r_[cols, d + cols, 2 * d + cols]]
+    for part, name in enumerate("qkv"):
+        assert rel(got_d[:, part * 64:(part + 1) * 64], want_d[:, part * 64:(part + 1) * 64]) < 1e-2, name
+    dv = dqkv.view(B, T, 3, H, 64)[:, :, 2].float().sum(1)
+    g = do.view(B, T, H, 64).float().sum(1)
+    assert rel(host(dv), host(g)) < 1e-2
+
+
 def test_rejects_unsupported_shapes():
     lib = library()
     t = torch.zeros(4096, dtype=torch.bfloat16, device="cuda")

@@ -88,6 +88,69 @@ def test_training_is_deterministic_and_learns_at_full_size(name):
     assert per_step[-1] < per_step[0] - 0.02  # six AdamW steps already lower the loss
 
 
+def against_the_checker(orc, cfg, seed):
+    """tg_batch of one sequence against the CPU checker on the same weights and tokens.  Returns the relative errors
+    (logits, flat gradient, worst parameter tensor, mean loss) of the device against the fp32 checker, and the
+    errors of the checker's own rounding variant (bf16 at the device's store points) against its fp32 self: the size
+    of the rounding noise this depth and width produce, measured rather than assumed."""
+    T, d = cfg["context"], cfg["d_model"]
+    oc = orc.model(cfg["depth"], T, 1, d, cfg["heads"])
+    with Native(ModelConfig(**cfg)) as engine:
+        assert engine.count == orc.parameter_count(oc)
+        w = weights(engine.count, cfg, seed)
+        rng = np.random.default_rng(5)
+        for name, offset, shape in orc.Layout(oc).entries:  # norm parameters off their defaults
+            if name.endswith(("_g", "_b")):
+                w[offset:offset + shape[0]] += rng.standard_normal(shape[0]).astype(np.float32) * 0.1
+        engine.set_weights(w)
+        x = zipf_bytes(T, 71).reshape(1, T)
+        y = np.roll(x, -1, axis=1)
+        logits, grad, losses = engine.batch(x, y)
+
+    def rel(a, b):
+        a, b = np.asarray(a, np.float64), np.asarray(b, np.float64)
+        return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-12))
+
+    def worst(g, want):
+        return max((rel(g[o:o + int(np.prod(s))], want[o:o + int(np.prod(s))]), name)
+                   for name, o, s in orc.Layout(oc).entries)
+
+    want_logits, want_grad, want_loss = orc.model_batch(oc, w, x, y)
+    rounding = orc.model(cfg["depth"], T, 1, d, cfg["heads"], emulate=True)
+    noisy_logits, noisy_grad, _ = orc.model_batch(rounding, w, x, y)
+    device = (rel(logits, want_logits), rel(grad, want_grad), worst(grad, want_grad),
+              abs(float(losses.mean()) - float(want_loss.mean())))
+    noise = (rel(noisy_logits, want_logits), rel(noisy_grad, want_grad), worst(noisy_grad, want_grad))
+    return device, noise
+
+
+def test_long_context_shape_against_the_checker(orc):
+    """Two blocks of the long-context model (d1024 H16 T4096: the widths, tile shapes and attention loop of
+    configs[4]; depth 2 and one sequence keep the CPU checker at a minute) through tg_batch against the checker:
+    logits and the flat gradient to 1e-2, every parameter tensor's gradient to 2e-2, mean loss to 3e-3; and no
+    further from the fp32 checker than bf16 rounding at the device's store points takes the checker itself."""
+    cfg = dict(CONFIGS["configs[4]"], depth=2, batch=1)
+    (logits, grad, worst, loss), noise = against_the_checker(orc, cfg, 99)
+    print(f"long-context shape: logits {logits:.3g}, gradient {grad:.3g}, worst tensor {worst}; rounding noise of the "
+          f"checker itself: logits {noise[0]:.3g}, gradient {noise[1]:.3g}, worst {noise[2]}", flush=True)
+    assert logits < 1e-2 and grad < 1e-2 and worst[0] < 2e-2 and loss < 3e-3
+    assert logits < 1.3 * noise[0] + 5e-4 and grad < 1.3 * noise[1] + 5e-4
+
+
+def test_headline_shape_against_the_rounding_checker(orc):
+    """The headline shape (d768 L12 H12 T1024, one sequence).  Twelve blocks of bf16 stores put the logits close to
+    the 1e-2 bar against the fp32 checker; how much of that is rounding is measured, not assumed: the checker's own
+    variant that rounds at the device's store points lands as far from its fp32 self.  (The two rounded computations
+    cannot be held to each other more tightly - a different summation order flips bf16 ties and they drift apart like
+    independent samples - so the bound is on the size of the error, not on the difference.)  An error on top of
+    rounding shows as a device error beyond 1.3 x that noise."""
+    cfg = dict(CONFIGS["configs[3]"], batch=1)
+    (logits, grad, worst, loss), noise = against_the_checker(orc, cfg, 3407)
+    print(f"headline shape: logits {logits:.3g}, gradient {grad:.3g}, worst tensor {worst}; rounding noise of the "
+          f"checker itself: logits {noise[0]:.3g}, gradient {noise[1]:.3g}, worst {noise[2]}", flush=True)
+    assert logits < 1.3 * noise[0] + 5e-4 and grad < 1.3 * noise[1] + 5e-4 and worst[0] < 1.3 * noise[2][0] + 1e-3
+
+
 def test_headline_shape_against_the_checker(orc):
     """One sequence of the headline model (d768 L12 H12 T1024, the shape bench.py times at batch 16) through
     tg_batch against the CPU checker on the same weights and tokens: logits and the flat gradient to 1e-2,

@@ -66,23 +66,24 @@ def test_the_reference_loads_a_checkpoint_the_library_wrote(tmp_path):
 
 def test_the_library_reads_a_checkpoint_the_reference_wrote(tmp_path):
     (weights, momentum, variance), sums = state(2)
-    scalars = np.array([40, 64, 1], np.int64)  # step 40 of 64: one step lies in the last max(1, ceil(64/100)) = 1
+    # step 64 of 64: the final-loss window is the last max(1, ceil(64 / 100)) = 1 step, and it has run: one batch
+    # with live sums (a state outside the window, such as step 40 with one batch, the reference refuses to save)
+    scalars = np.array([64, 64, 1], np.int64)
     reals = np.array([0.3, 0.04, 0.000004, 0.85, 0.95, 3.25])
     path = tmp_path / "reference.pt"
     status = ref.tgref_checkpoint_save(str(path).encode(), DEPTH, CONTEXT, C.c_int64(COUNT), pointer(weights),
                                        pointer(momentum), pointer(variance), pointer(scalars), pointer(reals), pointer(sums))
-    if status != 0:  # the reference validates the loss window: step 40 of 64 has no batch in it yet
-        assert b"final loss" in ref.tgref_io_error()
-        scalars[2] = 0
-        status = ref.tgref_checkpoint_save(str(path).encode(), DEPTH, CONTEXT, C.c_int64(COUNT), pointer(weights),
-                                           pointer(momentum), pointer(variance), pointer(scalars), pointer(reals),
-                                           pointer(sums))
     assert status == 0, ref.tgref_io_error()
+    early = np.array([40, 64, 1], np.int64)
+    assert ref.tgref_checkpoint_save(str(tmp_path / "early.pt").encode(), DEPTH, CONTEXT, C.c_int64(COUNT), pointer(weights),
+                                     pointer(momentum), pointer(variance), pointer(early), pointer(reals),
+                                     pointer(sums)) != 0
+    assert b"final loss" in ref.tgref_io_error()
     got = bridge.read_checkpoint(path)
     for name, want in (("weights", weights), ("momentum", momentum), ("variance", variance)):
         np.testing.assert_array_equal(got[name].view(np.uint32), want.view(np.uint32))
     np.testing.assert_array_equal(got["final_loss_sums"], sums)
-    assert got["step"] == 40 and got["train_seconds"] == 3.25 and got["final_loss_batches"] == scalars[2]
+    assert got["step"] == 64 and got["train_seconds"] == 3.25 and got["final_loss_batches"] == 1
     assert got["scheduler"] == dict(total_steps=64, warmup_fraction=0.3, initial_lr_fraction=0.04,
                                     final_lr_fraction=0.000004, low_momentum=0.85, high_momentum=0.95)
     # no width fields in the file: it reads as the reference's own network
@@ -94,13 +95,40 @@ def test_the_library_reads_a_checkpoint_the_reference_wrote(tmp_path):
     import torch
     ours = tmp_path / "ours.pt"
     bridge.write_checkpoint(ours, bridge.ModelConfig(d_model=16, heads=4, ffn=48, depth=DEPTH, context=CONTEXT), weights,
-                            momentum, variance, step=40, scheduler=bridge.OneCycle(64), train_seconds=3.25,
-                            final_loss_sums=sums, final_loss_batches=int(scalars[2]))
+                            momentum, variance, step=64, scheduler=bridge.OneCycle(64), train_seconds=3.25,
+                            final_loss_sums=sums, final_loss_batches=1)
     a, b = torch.load(path, weights_only=True), torch.load(ours, weights_only=True)
     assert set(a) == set(b) == {"model", "opt", "lr_scheduler", "trainer"}
     for section in a:
         for key, value in a[section].items():
             assert torch.equal(value, b[section][key]), (section, key)
+
+
+def test_the_library_refuses_width16_states_the_reference_would_refuse(tmp_path):
+    """A width-16 file is promised to load through the reference's reader, so the writer applies the reference's own
+    conditions (checkpoint.cpp:535-550) and writes nothing when they fail; the reference's writer refuses the same."""
+    (weights, momentum, variance), sums = state(3)
+    model = bridge.ModelConfig(d_model=16, heads=4, ffn=48, depth=DEPTH, context=CONTEXT)
+    good = dict(step=64, scheduler=bridge.OneCycle(64), train_seconds=1.0, final_loss_sums=sums, final_loss_batches=1)
+    bridge.write_checkpoint(tmp_path / "good.pt", model, weights, momentum, variance, **good)
+    cases = {
+        "window": dict(good, step=40),                          # one batch before the window has begun
+        "steps": dict(good, scheduler=bridge.OneCycle(0), step=0, final_loss_batches=0),
+        "past": dict(good, step=65),
+        "sums": dict(good, final_loss_sums=None, final_loss_batches=0),
+        "schedule": dict(good, scheduler=bridge.OneCycle(64, warmup_fraction=1.5)),
+    }
+    for name, fields_ in cases.items():
+        path = tmp_path / (name + ".pt")
+        with pytest.raises(RuntimeError):
+            bridge.write_checkpoint(path, model, weights, momentum, variance, **fields_)
+        assert not path.exists(), name
+    # the reference's writer on the first of them
+    early = np.array([40, 64, 1], np.int64)
+    reals = np.array([0.3, 0.04, 0.000004, 0.85, 0.95, 1.0])
+    assert ref.tgref_checkpoint_save(str(tmp_path / "ref.pt").encode(), DEPTH, CONTEXT, C.c_int64(COUNT), pointer(weights),
+                                     pointer(momentum), pointer(variance), pointer(early), pointer(reals),
+                                     pointer(sums)) != 0
 
 
 def summaries(path):

@@ -96,8 +96,10 @@ class OneCycle(C.Structure):
         (name, C.c_double) for name in ("warmup_fraction", "initial_lr_fraction", "final_lr_fraction",
                                         "low_momentum", "high_momentum")]
 
-    def __init__(self, total_steps):
-        super().__init__(total_steps, .3, .04, .000004, .85, .95)
+    def __init__(self, total_steps, warmup_fraction=.3, initial_lr_fraction=.04, final_lr_fraction=.000004,
+                 low_momentum=.85, high_momentum=.95):
+        super().__init__(total_steps, warmup_fraction, initial_lr_fraction, final_lr_fraction, low_momentum,
+                         high_momentum)
 
 
 class StepRates(C.Structure):
@@ -158,7 +160,7 @@ EVENTS_ABI = {
     "tg_crc32c": (C.c_uint32, [vp, sz]),
 }
 CLASSES = ("gemm_fwd", "gemm_dgrad", "gemm_wgrad", "attn_fwd", "attn_bwd", "layernorm_fwd", "layernorm_bwd",
-           "head", "other", "optimizer")
+           "head", "other", "optimizer", "gemm_fwd_gelu", "gemm_dgrad_gelu")
 
 
 def library_path():

@@ -697,7 +697,15 @@ float *scratch_on_current_device() {
 }
 } // namespace
 
-extern "C" size_t tgk_attn_bwd_static_max_rows(void) { return STATIC_BWD_ROWS; }
+// Also the set-up call: it looks up the array's address on the current device, so that a later tgk_attn_bwd_static
+// on this device (under stream capture, say) has nothing left to resolve.  A failed lookup is reported by that call.
+extern "C" size_t tgk_attn_bwd_static_max_rows(void) {
+    try {
+        (void)scratch_on_current_device();
+    } catch (const std::exception &) {
+    }
+    return STATIC_BWD_ROWS;
+}
 
 extern "C" int tgk_attn_bwd_static(hipStream_t stream, int B, int H, int T, int hd, const uint16_t *Q,
                                    const uint16_t *K, const uint16_t *V, int ld, const uint16_t *O, int ldo,

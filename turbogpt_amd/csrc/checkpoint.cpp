@@ -13,6 +13,7 @@
 #include "../../include/tg_checkpoint.h"
 #include "../../include/tg_model.h"
 
+#include <algorithm>
 #include <cerrno>
 #include <cstdio>
 #include <cstring>
@@ -360,6 +361,25 @@ void check_for_writing(const TgCheckpoint &c) {
         fail("final_loss_sums is missing");
     if (c.scheduler.total_steps < 0)
         fail("scheduler.total_steps is negative");
+    // A width-16 file is promised to load through the reference's load_training_state, which refuses what follows
+    // (checkpoint.cpp:535-550, optim.h:18-30): such a state is refused here, before anything is written.
+    if (m.d_model == 16 && m.heads == 4 && m.vocab == 256 && m.ffn == 48) {
+        const OneCycle &s = c.scheduler;
+        if (c.final_loss_positions != m.base.context)
+            fail("a width-16 checkpoint carries one final-loss sum per position (final_loss_positions = context)");
+        if (s.total_steps < 1 || c.step > uint64_t(s.total_steps))
+            fail("a width-16 checkpoint needs scheduler.total_steps >= 1 and step <= total_steps");
+        const int64_t total = s.total_steps, window = std::max<int64_t>(1, (total + 99) / 100);
+        const int64_t first = std::max<int64_t>(0, total - window);
+        if (int64_t(c.final_loss_batches) > std::max<int64_t>(0, int64_t(c.step) - first))
+            fail("final_loss_batches exceeds the steps of the final-loss window that have run");
+        const bool fractions = s.warmup_fraction > 0 && s.warmup_fraction < 1 && s.initial_lr_fraction > 0 &&
+                               s.initial_lr_fraction < 1 && s.final_lr_fraction > 0 &&
+                               s.final_lr_fraction <= s.initial_lr_fraction && s.low_momentum >= 0 && s.low_momentum < 1 &&
+                               s.high_momentum >= s.low_momentum && s.high_momentum < 1;
+        if (!fractions || s.warmup_fraction * s.total_steps - 1 == 0)
+            fail("a width-16 checkpoint needs a valid OneCycle schedule");
+    }
 }
 
 void write_checkpoint(const char *path, const TgCheckpoint &c) {

@@ -250,7 +250,7 @@ struct Engine {
             OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, d, b.o, d, w(p.attn_out), d, b.mid, d, x[l], d, nullptr, 0));
             OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, b.mid, w(p.ln2_g), wl(p.ln2_g), w(p.ln2_b), wl(p.ln2_b), b.n2,
                                  config.ln_eps));
-            OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, F, d, b.n2, d, w(p.mlp_up), d, b.u, F, nullptr, 0, b.a, F));
+            OP(TG_CLASS_GEMM_FWD_GELU, tgk_gemm_fwd(stream, M, F, d, b.n2, d, w(p.mlp_up), d, b.u, F, nullptr, 0, b.a, F));
             OP(TG_CLASS_GEMM_FWD, tgk_gemm_fwd(stream, M, d, F, b.a, F, w(p.mlp_down), F, x[l + 1], d, b.mid, d, nullptr, 0));
         }
         OP(TG_CLASS_LAYERNORM_FWD, tgk_layernorm_fwd(stream, M, d, x[c.depth], w(layout.lnf_g), wl(layout.lnf_g), w(layout.lnf_b),
@@ -298,7 +298,7 @@ struct Engine {
                 const TgLayerParameters &p = layout.layers[l];
                 LayerBuffers &b = layers[l];
                 bf16_t *in = s.g_x[l + 1], *mid = s.g_mid[l], *gu = s.g_u[l], *gqkv = s.g_qkv[l];
-                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, in, d, wt(p.mlp_down), d, gu, F, b.u, F));
+                OP(TG_CLASS_GEMM_DGRAD_GELU, tgk_gemm_dgrad_t(stream, M, d, F, in, d, wt(p.mlp_down), d, gu, F, b.u, F));
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, gu, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
                 OP(TG_CLASS_LAYERNORM_BWD, ln_rows(1 + 2 * l, b.mid, t1, p.ln2_g, in, mid));
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, d, mid, d, wt(p.attn_out), d, t1, d, nullptr, 0));
@@ -326,7 +326,7 @@ struct Engine {
                 // go out as one launch; for that the gradient entering the block (dh) survives the block's first
                 // half: LayerNorm 2 writes its sum with dh into dh_mid.
                 bf16_t *mid = s.dh_mid;
-                OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
+                OP(TG_CLASS_GEMM_DGRAD_GELU, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, du, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
                 OP(TG_CLASS_LAYERNORM_BWD, ln_rows(1 + 2 * l, b.mid, t1, p.ln2_g, dh, mid));
                 OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, d, mid, d, wt(p.attn_out), d, t1, d, nullptr, 0));
@@ -343,7 +343,7 @@ struct Engine {
                 continue;
             }
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, d, F, dh, d, b.a, F, g + p.mlp_down, F, 0, workspace, workspace_bytes));
-            OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
+            OP(TG_CLASS_GEMM_DGRAD_GELU, tgk_gemm_dgrad_t(stream, M, d, F, dh, d, wt(p.mlp_down), d, du, F, b.u, F));
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad(stream, M, F, d, du, F, b.n2, d, g + p.mlp_up, d, 0, workspace, workspace_bytes));
             OP(TG_CLASS_GEMM_DGRAD, tgk_gemm_dgrad_t(stream, M, F, d, du, F, wt(p.mlp_up), F, t1, d, nullptr, 0));
             OP(TG_CLASS_LAYERNORM_BWD, ln_rows(1 + 2 * l, b.mid, t1, p.ln2_g, dh, dh));

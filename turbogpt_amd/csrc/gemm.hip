@@ -581,6 +581,7 @@ TG_DEVICE void multiply_stage(f32x4 (&acc)[FM][FN][2][2], const unsigned char *s
     // A column = one 16-row B fragment against the 2 FM A fragments of its 32-k step.  The A fragments of both steps
     // are held (the second step's are read during the first), B fragments are read one column ahead.
     constexpr int AF = 2 * FM, BF = 2 * FN, COLUMNS = 2 * BF;
+    static_assert(BF >= AF, "the second step's A fragments are read while the first step's B columns are walked");
     const unsigned char *sa = slot, *sb = sa + TA::BYTES;
     bf16x8 af[2][AF], bfr[2];
 #pragma unroll

@@ -18,6 +18,7 @@
 #include "tg_model.h"
 #include "tg_runtime.h"
 
+#include <limits>
 #include <algorithm>
 #include <array>
 #include <chrono>
@@ -135,29 +136,59 @@ std::vector<float> initial_weights_width16(const Config &c, int64_t count) {
     return w;
 }
 
-std::string sample(Engine *engine, const TgModelConfig &m) {
-    const std::string prompt = "The ";
-    std::vector<uint8_t> sequence(prompt.begin(), prompt.end());
-    std::mt19937 random(unsigned(m.base.seed));
-    std::vector<float> logits(256);
-    std::array<int, 256> tokens{};
-    for (int step = 0; step < 64; ++step) {
-        std::vector<uint8_t> context(size_t(m.base.context), 0);
-        const size_t have = std::min(sequence.size(), context.size());
-        std::copy(sequence.end() - long(have), sequence.end(), context.end() - long(have));
-        check(tg_predict(engine, context.data(), logits.data()));
-        std::iota(tokens.begin(), tokens.end(), 0);
-        std::partial_sort(tokens.begin(), tokens.begin() + 10, tokens.end(),
-                          [&](int a, int b) { return logits[size_t(a)] > logits[size_t(b)]; });
-        std::array<double, 10> p{};
-        for (int k = 0; k < 10; ++k)
-            p[size_t(k)] = std::exp(double(logits[size_t(tokens[size_t(k)])]) - double(logits[size_t(tokens[0])]));
-        std::discrete_distribution<int> choose(p.begin(), p.end());
-        sequence.push_back(uint8_t(tokens[size_t(choose(random))]));
+// The ten likeliest next bytes, likeliest first, with their logits: one pass with a small sorted list.
+struct Candidate {
+    int byte;
+    float logit;
+};
+std::array<Candidate, 10> likeliest(const std::vector<float> &logits) {
+    std::array<Candidate, 10> best;
+    best.fill({0, -std::numeric_limits<float>::infinity()});
+    for (int byte = 0; byte < 256; ++byte) {
+        const float logit = logits[size_t(byte)];
+        if (!(logit > best.back().logit))
+            continue;
+        size_t place = best.size() - 1;
+        for (; place > 0 && logit > best[place - 1].logit; --place)
+            best[place] = best[place - 1];
+        best[place] = {byte, logit};
     }
-    std::string text;
-    for (uint8_t c : sequence)
-        text += (c >= 32 && c < 127 && c != '"' && c != '\\') ? char(c) : '.';
+    return best;
+}
+
+// Text continued byte by byte from the trained model through tg_predict (the slot of sampling.cpp:10-42): the window
+// holds the last `context` bytes, right-aligned behind zeros; each byte is drawn from the softmax over the ten
+// likeliest, by inverting the cumulative weights at a uniform number from a generator seeded with the model's seed.
+std::string sample(Engine *engine, const TgModelConfig &m) {
+    const int generated = 64;
+    std::vector<uint8_t> window(size_t(m.base.context), 0);
+    std::string text = "The ";
+    auto push = [&](uint8_t byte) {
+        std::move(window.begin() + 1, window.end(), window.begin());
+        window.back() = byte;
+    };
+    for (char c : text)
+        push(uint8_t(c));
+    uint64_t state = uint64_t(m.base.seed) * 0x9e3779b97f4a7c15ull + 1;
+    auto uniform = [&]() { // xorshift64*: 53 random bits as a number in [0, 1)
+        state ^= state >> 12, state ^= state << 25, state ^= state >> 27;
+        return double((state * 0x2545f4914f6cdd1dull) >> 11) * (1.0 / 9007199254740992.0);
+    };
+    std::vector<float> logits(256);
+    for (int n = 0; n < generated; ++n) {
+        check(tg_predict(engine, window.data(), logits.data()));
+        const auto best = likeliest(logits);
+        double weight[10], total = 0;
+        for (size_t k = 0; k < best.size(); ++k)
+            total += weight[k] = std::exp(double(best[k].logit) - double(best[0].logit));
+        double left = uniform() * total;
+        size_t pick = 0;
+        while (pick + 1 < best.size() && left >= weight[pick])
+            left -= weight[pick++];
+        const uint8_t byte = uint8_t(best[pick].byte);
+        push(byte);
+        text += (byte >= 32 && byte < 127 && byte != '"' && byte != '\\') ? char(byte) : '.';
+    }
     return text;
 }
 
