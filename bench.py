@@ -29,7 +29,7 @@ CONFIGS = {3: dict(D=768, L=12, H=12, T=1024, B=16), 4: dict(D=1024, L=24, H=16,
 D, L, H, T, B = (CONFIGS[3][k] for k in "DLHTB")
 F = 4 * D
 M = B * T
-TRAFFIC_PROFILE = "profiles/gemm64_kc_kc_hbm_traffic.md"
+TRAFFIC_PROFILE = "profiles/gemm256_plain_residual_hbm_traffic.md"
 
 
 def select_config(index):
@@ -285,9 +285,9 @@ def kernel_sweeps(out):
 
 def traffic_probe():
     """For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: one plain copy of known size (256 MiB in,
-    256 MiB out: the calibration dispatch) followed by one launch of each forward block projection
-    and of each dgrad (on transposed weights), as the engine runs them - the eight uses per layer of the
-    kernel that `roofline` describes."""
+    256 MiB out: the calibration dispatch) followed by the six launches per layer of the kernel that
+    `roofline` describes, through the entries the engine uses: QKV, attention-out (+ residual) and MLP-down
+    (+ residual) forward on the weights, then MLP-up, attention-out and QKV dgrad on the transposed copies."""
     import torch
     from turbogpt_amd.bridge import check, library
     lib = library()
@@ -297,22 +297,31 @@ def traffic_probe():
     torch.cuda.synchronize()
     dst.copy_(src)
     torch.cuda.synchronize()
-    shapes = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
-    for k, n in shapes:
-        x = torch.randn(M, k, device="cuda").bfloat16()
-        w = torch.randn(n, k, device="cuda").bfloat16()
-        wt = w.t().contiguous()
-        dy = torch.randn(M, n, device="cuda").bfloat16()
-        y = torch.empty(M, n, device="cuda", dtype=torch.bfloat16)
-        dx = torch.empty(M, k, device="cuda", dtype=torch.bfloat16)
+    bf16 = torch.bfloat16
+    forward = [(D, 3 * D, False), (D, D, True), (F, D, True)]  # (K, N, residual)
+    for k, n, residual in forward:
+        x = torch.randn(M, k, device="cuda").to(bf16)
+        w = (torch.randn(n, k, device="cuda") * 0.02).to(bf16)
+        r = torch.randn(M, n, device="cuda").to(bf16) if residual else None
+        y = torch.empty(M, n, device="cuda", dtype=bf16)
         torch.cuda.synchronize()
-        check(lib.tgk_gemm_fwd(stream, M, n, k, x.data_ptr(), k, w.data_ptr(), k, y.data_ptr(), n, None, 0, None, 0))
+        check(lib.tgk_gemm_fwd(stream, M, n, k, x.data_ptr(), k, w.data_ptr(), k, y.data_ptr(), n,
+                               r.data_ptr() if residual else None, n if residual else 0, None, 0))
+        torch.cuda.synchronize()
+    dgrad = [(D, F), (D, D), (D, 3 * D)]  # (K = width of dx, N = width of dy)
+    for k, n in dgrad:
+        dy = torch.randn(M, n, device="cuda").to(bf16)
+        wt = (torch.randn(k, n, device="cuda") * 0.02).to(bf16)
+        dx = torch.empty(M, k, device="cuda", dtype=bf16)
         torch.cuda.synchronize()
         check(lib.tgk_gemm_dgrad_t(stream, M, n, k, dy.data_ptr(), n, wt.data_ptr(), n, dx.data_ptr(), k, None, 0))
         torch.cuda.synchronize()
     print(json.dumps({"probe": "traffic", "copy_bytes_each_way": 1 << 28,
-                      "order": "per shape (K, N): forward, then dgrad", "shapes": shapes,
-                      "algorithmic_bytes_per_launch": [2 * (M * k + n * k + M * n) for k, n in shapes]}))
+                      "order": "forward (K, N, residual) x 3, then dgrad (K, N) x 3",
+                      "forward": forward, "dgrad": dgrad,
+                      "algorithmic_bytes_per_launch":
+                          [2 * (M * k + n * k + M * n * (2 if r else 1)) for k, n, r in forward] +
+                          [2 * (M * n + n * k + M * k) for k, n in dgrad]}))
 
 
 def main():
@@ -323,7 +332,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernels", action="store_true", help="also print the isolated kernel sweeps to stderr")
     ap.add_argument("--traffic-probe", action="store_true",
-                    help="run only the copy + forward GEMM dispatches used to read HBM traffic counters")
+                    help="run only the copy and the six dominant GEMM dispatches used to read HBM traffic counters")
     ap.add_argument("--config", type=int, default=3, choices=sorted(CONFIGS),
                     help="3: d768 L12 T1024 B16 (the metric's configuration); 4: d1024 L24 T4096 B4")
     args = ap.parse_args()
