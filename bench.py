@@ -380,15 +380,16 @@ def main():
     traffic, traffic_source = hbm_traffic_per_launch() if args.config == 3 else (None, "not measured for this configuration")
     # Dominant MFMA kernel: the forward block projections and input gradients with a plain or residual epilogue, six
     # launches per layer - QKV, attention-out and MLP-down forward (on the weights), MLP-up, attention-out and QKV dgrad
-    # (on the transposed copies).  Widths that 192 and 384 divide run them on gemm256_kernel<EpilogueBf16As<0|1>>
-    # (256 x 192 tiles), others on gemm64_kernel<128,128|192,true,true,EpilogueBf16As<0|1>>.
+    # (on the transposed copies).  Widths that 192 and 384 divide run them on gemm256_kernel<192,3,...> (256 x 192
+    # tiles), widths that 128 and 256 divide on gemm256_kernel<128,4,...> (256 x 128), others on gemm64_kernel.
     fwd_ms, fwd_launches = profile["gemm_fwd"]
     dgrad_ms, dgrad_launches = profile["gemm_dgrad"]
     launch_ms = (fwd_ms + dgrad_ms) / (fwd_launches + dgrad_launches)
     qkv, out, up, down = gemm_flops()
     flops_per_launch = (2 * qkv + 2 * out + up + down) / 6
     achieved = flops_per_launch / (launch_ms * 1e-3) / 1e12
-    kernel = ("gemm256_kernel<EpilogueBf16As<0|1>> (256x192 tiles, one wave per SIMD)" if D % 384 == 0 else
+    kernel = ("gemm256_kernel<192,3,EpilogueBf16As<0|1>> (256x192 tiles, one wave per SIMD)" if D % 384 == 0 else
+              "gemm256_kernel<128,4,EpilogueBf16As<0|1>> (256x128 tiles, one wave per SIMD)" if D % 256 == 0 else
               "gemm64_kernel<128,128|192,true,true,EpilogueBf16As<0|1>>")
     ms_per_step = seconds / args.steps * 1e3
     result = {

@@ -367,6 +367,42 @@ def test_rejects_bad_shapes_without_launching():
     sync()
 
 
+@pytest.mark.parametrize("M,N,K,residual", [(16384, 1024, 256, False), (16384, 1024, 512, True), (8192, 2048, 1024, False),
+                                          (16384, 3072, 1024, True), (16384, 1024, 4096, False)])
+def test_256x128_tiles_rows_sampled(orc, M, N, K, residual):
+    """The widths of configs[4] (multiples of 128 and 256 that 192 does not divide) run on 256 x 128 tiles whose
+    epilogue buffers lie in a ring slot: forward with and without a residual and the input gradient on the transposed
+    weight, one to six tiles per block and one to sixteen periods per tile, against the checker on sampled rows and bit
+    for bit against the kernels for k-strided weights, which sum in the same order."""
+    lib = library()
+    rng = np.random.default_rng(M + N + K)
+    x, xh = to_bf16_device(rng.standard_normal((M, K)))
+    w, wh = to_bf16_device(rng.standard_normal((N, K)) / np.sqrt(K))
+    r, rh = to_bf16_device(rng.standard_normal((M, N)))
+    rows = np.sort(rng.choice(M, 64, replace=False))
+    y, _ = run_fwd(x, w, residual=r if residual else None)
+    want = orc.gemm_fwd(xh[rows], wh, residual=rh[rows] if residual else None)
+    assert rel(host(y)[rows], want) < 1e-2
+    assert np.mean(host(y)[rows] == orc.gemm_fwd(xh[rows], wh, residual=rh[rows] if residual else None, emulate=True)) > 0.99
+    yt = torch.empty_like(y)
+    wt = w.t().contiguous()
+    check(lib.tgk_gemm_fwd_t(stream(), M, N, K, x.data_ptr(), K, wt.data_ptr(), N, yt.data_ptr(), N,
+                             r.data_ptr() if residual else None, N if residual else 0, None, 0))
+    sync()
+    assert torch.equal(yt, y)  # 32-k stages on the k-strided weight: same products, same summation order
+    # input gradient: dX[M][K] = dY[M][N] W[N][K], tiled over (M, K) and reduced over N
+    dy, dyh = to_bf16_device(rng.standard_normal((M, N)))
+    w2, w2h = to_bf16_device(rng.standard_normal((N, K)) / np.sqrt(N))
+    dx = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+    dxt = torch.empty_like(dx)
+    w2t = w2.t().contiguous()
+    check(lib.tgk_gemm_dgrad_t(stream(), M, N, K, dy.data_ptr(), N, w2t.data_ptr(), N, dxt.data_ptr(), K, None, 0))
+    check(lib.tgk_gemm_dgrad(stream(), M, N, K, dy.data_ptr(), N, w2.data_ptr(), K, dx.data_ptr(), K, None, 0))
+    sync()
+    assert rel(host(dxt)[rows], orc.gemm_dgrad(dyh[rows], w2h)) < 1e-2
+    assert torch.equal(dxt, dx)
+
+
 @pytest.mark.parametrize("N,K", [(2304, 768), (768, 768), (3072, 768), (768, 3072)])
 def test_full_size_sweep_rows_sampled(orc, N, K):
     """BASELINE config 2 at M = 16384: the checker covers a sample of output rows/columns."""

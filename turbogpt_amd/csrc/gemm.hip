@@ -745,27 +745,40 @@ TG_DEVICE uint32_t kc64_frag16_offset(int row0, int ks, int lane) { // TileKC64:
     const int row = row0 + (lane & 15), chunk = (ks * 4 + (lane >> 4)) ^ ((row >> 1) & 7);
     return uint32_t(row * 128 + chunk * 16);
 }
-// ---- 256 x 192 tiles, one wave per SIMD: forward and input-gradient products with a long or plain epilogue ------
-// C = A B^T with both operands k-contiguous, a 256 x 192 tile per block, four waves of 128 x 96 outputs each, one
+// ---- 256-row tiles, one wave per SIMD: forward and input-gradient products with a long or plain epilogue -------------
+// C = A B^T with both operands k-contiguous, a 256 x BN tile per block, four waves of 128 x BN/2 outputs each, one
 // block per compute unit.  What bounds these products is a compute unit's copy path: bytes per flop, whole
-// cache lines per request, and how many requests it keeps in flight.  Hence: 9.1 bytes per kFLOP without relying on
-// another block's lines in L1; 64 k per stage (every request a whole 128-byte line); and rings of different depth for
-// the two operands - three slots for A (activations, streamed from beyond the L2: a copy has two stages to land) and
-// two for B (the weights, mostly L2 hits: one stage), 144 KB of LDS.  With a lone wave per SIMD the fragments of the
+// cache lines per request, and how many requests it keeps in flight.  Hence: 9.1 bytes per kFLOP at BN = 192 without
+// relying on another block's lines in L1; 64 k per stage (every request a whole 128-byte line); and rings of different
+// depth for the two operands - RA slots for A (activations, streamed from beyond the L2: a copy has two stages to
+// land) and two for B (the weights, mostly L2 hits: one stage).  With a lone wave per SIMD the fragments of the
 // next 32-k step are read into a second register set between the matrix instructions of the current one:
 //   first half of stage g : matrix instructions on (g, k 0..31), fragment reads of (g, k 32..63)
 //   wait (all but A's youngest stage), barrier: stage g + 1 is visible, nobody reads stage g's slots any more
-//   second half           : matrix instructions on (g, k 32..63), copies of B's stage g + 2 and A's stage g + 3,
+//   second half           : matrix instructions on (g, k 32..63), copies of B's stage g + 2 and A's stage g + RA,
 //                           fragment reads of (g + 1, k 0..31)
-// The loop is unrolled over six stages (the rings' common period): the reduced dimension is a multiple of 384.
-template <class Epilogue>
+// The loop is unrolled over the rings' common period P, so that every LDS address is a constant, and the reduced
+// dimension is a multiple of 64 P.  Two instantiations:
+//   BN = 192, RA = 3 (P = 6, 144 KB of rings + 8 KB for the epilogue): widths that 192 and 384 divide;
+//   BN = 128, RA = 4 (P = 4, 160 KB of rings: all of the LDS): widths that 128 and 256 divide (d_model 1024).  Three
+//   slots would do for A as far as latency goes - the fourth only makes the period a power of two.  The epilogue's
+//   buffers then lie in the first 8 KB of the A slot that the tile's last stage leaves, and the two copies per wave that
+//   refill those rows are held back until the wave's epilogue is over (each wave then copies the rows under its own
+//   buffer, so no barrier is needed; in their place copies 2 and 3 of the stage go out twice, which keeps the loop
+//   free of branches and every wait count fixed).
+template <int BN, int RA, class Epilogue>
 __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restrict__ A, int lda,
-                                                       const bf16_t *__restrict__ B, int ldb, int k_sixes,
+                                                       const bf16_t *__restrict__ B, int ldb, int k_periods,
                                                        int tiles_n, int tiles_total, int xcd_cols,
                                                        Epilogue epilogue) {
-    constexpr int BM = 256, BN = 192;
+    constexpr int BM = 256;
+    constexpr int P = RA % 2 ? 2 * RA : RA; // stages per period of the two rings (RA slots for A, two for B)
     constexpr int WM = BM / 2, WN = BN / 2, FM = WM / 32, FN = WN / 32, AF = 2 * FM, BF = 2 * FN, MFMAS = AF * BF;
-    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, B_RING = 3 * A_BYTES, BUFFERS = B_RING + 2 * B_BYTES;
+    constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, B_RING = RA * A_BYTES, BUFFERS = B_RING + 2 * B_BYTES;
+    // Where the rings fill the LDS, the epilogue's four transposition buffers (8 KB) lie in the first rows of the A slot
+    // that a tile's last stage leaves, and the two copies per wave that would refill those rows wait for the epilogue.
+    constexpr bool ALIAS = BUFFERS + 4 * 2048 > 160 * 1024;
+    static_assert(!ALIAS || (P == RA && BUFFERS <= 160 * 1024), "the aliased buffers assume the last stage's slot is the ring's last");
     constexpr int LA = BM * 128 / 4096, LB = BN * 128 / 4096, LOADS = LA + LB; // copies per wave and stage
     constexpr int READ_EVERY = MFMAS / (AF + BF), COPY_EVERY = MFMAS / LOADS;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -822,7 +835,7 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
     tile_origin(blockIdx.x, pa_at, pb_at);
     a_next = pa_at, b_next = pb_at;
     prepare_next(blockIdx.x + stride);
-    // stages 0 and 1 of both, then A's stage 2 (so that A's youngest stage is the last one issued, as in the loop)
+    // stages 0 and 1 of both, then A's further stages (so that A's youngest stages are the last ones issued, as in the loop)
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
 #pragma unroll
@@ -834,9 +847,12 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
         pa_at += pa_step, pb_at += pb_step;
     }
 #pragma unroll
-    for (int n = 0; n < LA; ++n)
-        copy_a(n, 2);
-    pa_at += pa_step;
+    for (int s = 2; s < RA; ++s) {
+#pragma unroll
+        for (int n = 0; n < LA; ++n)
+            copy_a(n, s);
+        pa_at += pa_step;
+    }
 
     // ---- consumer ----------------------------------------------------------------------------------------------------
     uint32_t fa_at[2], fa_far[2], fb_at[2]; // fragment 0 of either 32-k step; fragment i lies 2048 i bytes further on
@@ -849,20 +865,20 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
     auto read_fragment = [&](bf16x8 (&fa)[AF], bf16x8 (&fb)[BF], int slot_a, int slot_b, int ks, int f)
                              __attribute__((always_inline)) {
         if (f < AF)
-            fa[f] = slot_a == 2 ? *reinterpret_cast<const bf16x8 *>(smem + fa_far[ks] + f * 2048)
+            fa[f] = slot_a >= 2 ? *reinterpret_cast<const bf16x8 *>(smem + fa_far[ks] + (slot_a - 2) * A_BYTES + f * 2048)
                                 : *reinterpret_cast<const bf16x8 *>(smem + fa_at[ks] + slot_a * A_BYTES + f * 2048);
         else
             fb[f - AF] = *reinterpret_cast<const bf16x8 *>(smem + fb_at[ks] + slot_b * B_BYTES + (f - AF) * 2048);
     };
     f32x4 acc[FM][FN][2][2];
-    bool last_six = k_sixes == 1; // the consumer is in a tile's last six stages
+    bool last_period = k_periods == 1; // the consumer is in a tile's last period of stages
     bool behind_epilogue = false;
-    static_assert(LA + FM * FN * Epilogue::MEMORY_OPS_PER_BLOCK < 64, "the wait count has six bits");
+    static_assert(LA + FM * FN * Epilogue::MEMORY_OPS_PER_BLOCK + (ALIAS ? 2 : 0) < 64, "the wait count has six bits");
     // One 32-k step on `cur`; meanwhile the fragments of (next slots, next_ks) are read into `next`, and, in a
     // stage's second half, the copies go out: B first, A behind it (so that a wait can leave A's youngest stage out).
     auto half = [&](auto copy_tag, int next_a_slot, int next_b_slot, int next_ks, int copy_a_slot, int copy_b_slot,
-                    const bf16x8 (&cur_a)[AF], const bf16x8 (&cur_b)[BF], bf16x8 (&next_a)[AF], bf16x8 (&next_b)[BF])
-                    __attribute__((always_inline)) {
+                    bool hold_back, const bf16x8 (&cur_a)[AF], const bf16x8 (&cur_b)[BF], bf16x8 (&next_a)[AF],
+                    bf16x8 (&next_b)[BF]) __attribute__((always_inline)) {
         constexpr bool COPY = decltype(copy_tag)::value;
 #pragma unroll
         for (int j = 0; j < BF; ++j)
@@ -879,27 +895,29 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
                     const int n = q / COPY_EVERY;
                     if (n < LB)
                         copy_b(n, copy_b_slot);
+                    else if (ALIAS && n - LB < 2) // held back: the rows under the epilogue's buffers; copy 2 or 3 goes twice instead
+                        copy_a(hold_back ? n - LB + 2 : n - LB, copy_a_slot);
                     else
                         copy_a(n - LB, copy_a_slot);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
     };
-    // stage g = STAGE (mod 6): A slot g % 3, B slot g % 2
+    // stage g = STAGE (mod P): A slot g % RA, B slot g % 2
     auto stage = [&](auto stage_tag, bf16x8 (&fa0)[AF], bf16x8 (&fb0)[BF], bf16x8 (&fa1)[AF], bf16x8 (&fb1)[BF])
                      __attribute__((always_inline)) {
-        constexpr int G = decltype(stage_tag)::value, SA = G % 3, SB = G % 2;
-        // In a tile's last six stages the producers cross into the next tile: A with the copies of stage 3 (three
-        // stages ahead), B with those of stage 4.  Selects, not branches.
-        if (G == 3 && last_six)
+        constexpr int G = decltype(stage_tag)::value, SA = G % RA, SB = G % 2;
+        // In a tile's last period the producers cross into the next tile: A with the copies of stage P - RA (RA
+        // stages ahead), B with those of stage P - 2.  Selects, not branches.
+        if (G == P - RA && last_period)
             pa_at = a_next, pa_step = next_step;
-        if (G == 4 && last_six)
+        if (G == P - 2 && last_period)
             pb_at = b_next, pb_step = next_step;
-        half(std::false_type{}, SA, SB, 1, 0, 0, fa0, fb0, fa1, fb1);
+        half(std::false_type{}, SA, SB, 1, 0, 0, false, fa0, fb0, fa1, fb1);
         // Everything but A's youngest stage has landed.  A wave's loads and stores retire in order through one counter;
         // behind a tile's epilogue its loads and stores are the youngest operations, and their number is known.
         if (G == 0 && behind_epilogue)
-            wait_vmcnt<LA + FM * FN * Epilogue::MEMORY_OPS_PER_BLOCK>();
+            wait_vmcnt<LA + FM * FN * Epilogue::MEMORY_OPS_PER_BLOCK + (ALIAS ? 2 : 0)>();
         else
             wait_vmcnt<LA>();
         if (G == 0)
@@ -908,7 +926,7 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         // copies: B's stage g + 2 into B slot g % 2, A's stage g + 3 into A slot g % 3 (the slots this stage leaves)
-        half(std::true_type{}, (SA + 1) % 3, SB ^ 1, 0, SA, SB, fa1, fb1, fa0, fb0);
+        half(std::true_type{}, (SA + 1) % RA, SB ^ 1, 0, SA, SB, ALIAS && G == P - 1 && last_period, fa1, fb1, fa0, fb0);
         pa_at += pa_step, pb_at += pb_step;
     };
     const bf16x8 zeros = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -924,23 +942,25 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
                                  : "v"(zeros)); // zeroed in place, wait states included (see wgrad_list_kernel)
     };
     bf16x8 fa0[AF], fb0[BF], fa1[AF], fb1[BF];
-    wait_vmcnt<LA + LOADS>(); // stage 0
+    wait_vmcnt<(RA - 1) * LA + LB>(); // stage 0
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int f = 0; f < AF + BF; ++f)
         read_fragment(fa0, fb0, 0, 0, 0, f);
-    unsigned char *mine = smem + BUFFERS + wave * 2048;
-    int item = blockIdx.x, sixes_left = k_sixes;
+    unsigned char *mine = smem + (ALIAS ? (RA - 1) * A_BYTES : BUFFERS) + wave * 2048;
+    int item = blockIdx.x, periods_left = k_periods;
     clear();
     for (;;) {
         stage(std::integral_constant<int, 0>{}, fa0, fb0, fa1, fb1);
         stage(std::integral_constant<int, 1>{}, fa0, fb0, fa1, fb1);
         stage(std::integral_constant<int, 2>{}, fa0, fb0, fa1, fb1);
         stage(std::integral_constant<int, 3>{}, fa0, fb0, fa1, fb1);
-        stage(std::integral_constant<int, 4>{}, fa0, fb0, fa1, fb1);
-        stage(std::integral_constant<int, 5>{}, fa0, fb0, fa1, fb1);
-        if (--sixes_left) {
-            last_six = sixes_left == 1;
+        if constexpr (P == 6) {
+            stage(std::integral_constant<int, 4>{}, fa0, fb0, fa1, fb1);
+            stage(std::integral_constant<int, 5>{}, fa0, fb0, fa1, fb1);
+        }
+        if (--periods_left) {
+            last_period = periods_left == 1;
             continue;
         }
         asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7"); // the compiler does not know that matrix instructions wrote the accumulators
@@ -951,12 +971,24 @@ __global__ __launch_bounds__(256, 1) void gemm256_kernel(const bf16_t *__restric
             load_aux_pair<FM, FN>(epilogue, 0, m0 + wm, n0 + wn, lane, aux);
         staged_store_bf16<FM, FN>(acc, aux, mine, epilogue, m0 + wm, n0 + wn, lane);
         behind_epilogue = true; // the stores stay in flight under the next tile's first stage
+        if (ALIAS) {
+            // the two copies held back in the last stage, as the rows that lie under this wave's own buffer (rows 16 w
+            // to 16 w + 15 of the stage: nobody else's buffer is touched, so no barrier); the producer has moved on
+            // by one stage since
+            __builtin_amdgcn_s_waitcnt(0xc07f); // this wave's reads of its buffer have returned
+#pragma unroll
+            for (int n = 0; n < 2; ++n) { // 1 KB piece 2 w + n of the stage: its rows' swizzle term goes by n, not by w
+                const int chunk = (lane & 7) ^ ((n * 4 + (lane >> 4)) & 7);
+                async_copy16(smem_base + uint32_t((RA - 1) * A_BYTES + (2 * wave + n) * 1024),
+                             pa_at - pa_step + int64_t(wave + n) * 8 * lda * 2, uint32_t(copy_row * lda + chunk * 8) * 2);
+            }
+        }
         item += stride;
         if (item >= tiles_total)
             break;
         prepare_next(item + stride);
-        sixes_left = k_sixes;
-        last_six = k_sixes == 1;
+        periods_left = k_periods;
+        last_period = k_periods == 1;
         clear();
     }
     wait_vmcnt<0>();
@@ -1576,21 +1608,28 @@ void launch_gemm64(hipStream_t stream, Tile tile, const bf16_t *A, int lda, cons
         launch_gemm64_tile<128, AKC, BKC>(stream, A, lda, B, ldb, M, N, K, splits, epilogue);
 }
 
-// The 256 x 192 kernel takes products with a plain or residual epilogue whose tiles fill the compute units a whole
+// The 256-row kernels take products with a plain or residual epilogue whose tiles fill the compute units a whole
 // number of times (or nearly): one block per unit, nothing to cover a tail or a long epilogue (the GELU epilogues
 // stay with gemm64_kernel, where the second block of a unit multiplies meanwhile).
-bool takes_256x192(int M, int N, int K, int mode) {
-    if (M % 256 || N % 192 || K % 384 || (mode != EPI_PLAIN && mode != EPI_RESIDUAL))
+bool takes_256(int M, int N, int K, int mode, int bn, int k_period) {
+    if (M % 256 || N % bn || K % k_period || (mode != EPI_PLAIN && mode != EPI_RESIDUAL))
         return false;
-    const int tiles = (M / 256) * (N / 192), units = compute_units();
+    const int tiles = (M / 256) * (N / bn), units = compute_units();
     const int rounds = (tiles + units - 1) / units;
     return tiles * 10 >= rounds * units * 9; // at least 90 % of the last round filled
 }
-template <class Epilogue>
+bool takes_256x192(int M, int N, int K, int mode) {
+    return takes_256(M, N, K, mode, 192, 384);
+}
+bool takes_256x128(int M, int N, int K, int mode) { // where the 192-wide tile does not fit
+    return !takes_256x192(M, N, K, mode) && takes_256(M, N, K, mode, 128, 256);
+}
+template <int BN = 192, int RA = 3, class Epilogue>
 void launch_gemm256(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
                     const Epilogue &epilogue) {
-    auto kernel = gemm256_kernel<Epilogue>;
-    constexpr size_t lds = 3 * 256 * 128 + 2 * 192 * 128 + 4 * 2048;
+    auto kernel = gemm256_kernel<BN, RA, Epilogue>;
+    constexpr size_t rings = RA * 256 * 128 + 2 * BN * 128, lds = rings + 4 * 2048 > 160 * 1024 ? rings : rings + 4 * 2048;
+    constexpr int P = RA % 2 ? 2 * RA : RA;
     static std::atomic<bool> configured[MAX_DEVICES];
     const int device = current_device();
     if (!configured[device].load(std::memory_order_acquire)) {
@@ -1599,10 +1638,10 @@ void launch_gemm256(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *
                   "gemm LDS size: ");
         configured[device].store(true, std::memory_order_release);
     }
-    const int tiles_m = M / 256, tiles_n = N / 192, tiles = tiles_m * tiles_n;
+    const int tiles_m = M / 256, tiles_n = N / BN, tiles = tiles_m * tiles_n;
     const int units = compute_units(), blocks = tiles < units ? tiles : units;
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, A, lda, B, ldb, K / 384, tiles_n, tiles,
-                       xcd_columns(tiles_m, tiles_n, 256, 192, K, blocks), epilogue);
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, A, lda, B, ldb, K / (64 * P), tiles_n, tiles,
+                       xcd_columns(tiles_m, tiles_n, 256, BN, K, blocks), epilogue);
     check_hip(hipGetLastError(), "gemm launch: ");
 }
 void launch_gemm256_bf16(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
@@ -1611,6 +1650,14 @@ void launch_gemm256_bf16(hipStream_t stream, const bf16_t *A, int lda, const bf1
         launch_gemm256(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_RESIDUAL>{e});
     else
         launch_gemm256(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_PLAIN>{e});
+}
+// 256 x 128 tiles, A ring of four slots (period of four stages: reduced dimensions that 256 divides)
+void launch_gemm256x128_bf16(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
+                             const EpilogueBf16 &e) {
+    if (e.mode == EPI_RESIDUAL)
+        launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_RESIDUAL>{e});
+    else
+        launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_PLAIN>{e});
 }
 
 // bf16 epilogues of the 64-k kernel: one instantiation per mode
@@ -1668,6 +1715,8 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
         }
         if (takes_256x192(M, N, K, e.mode))
             launch_gemm256_bf16(stream, X, ldx, W, ldw, M, N, K, e);
+        else if (takes_256x128(M, N, K, e.mode))
+            launch_gemm256x128_bf16(stream, X, ldx, W, ldw, M, N, K, e);
         else if (takes_64(tile, K))
             launch_gemm64_bf16<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, e);
         else
@@ -1740,6 +1789,8 @@ extern "C" int tgk_gemm_dgrad_t(hipStream_t stream, int M, int N, int K, const u
         // C[m][i] = sum_o dY[m][o] Wt[i][o]: the forward product with (rows, reduced) = (K, N)
         if (takes_256x192(M, K, N, e.mode))
             launch_gemm256_bf16(stream, dY, lddy, Wt, ldwt, M, K, N, e);
+        else if (takes_256x128(M, K, N, e.mode))
+            launch_gemm256x128_bf16(stream, dY, lddy, Wt, ldwt, M, K, N, e);
         else if (takes_64(tile, N))
             launch_gemm64_bf16<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, e);
         else
