@@ -371,8 +371,8 @@ def test_rejects_bad_shapes_without_launching():
                                           (16384, 3072, 1024, True), (16384, 1024, 4096, False)])
 def test_256x128_tiles_rows_sampled(orc, M, N, K, residual):
     """The widths of configs[4] (multiples of 128 and 256 that 192 does not divide) run on 256 x 128 tiles whose
-    epilogue buffers lie in a ring slot: forward with and without a residual and the input gradient on the transposed
-    weight, one to six tiles per block and one to sixteen periods per tile, against the checker on sampled rows and bit
+    epilogue buffers lie in a ring slot: forward with every epilogue and the input gradient on the transposed weight,
+    plain and times GELU', one to six tiles per block and one to sixteen periods per tile, against the checker on sampled rows and bit
     for bit against the kernels for k-strided weights, which sum in the same order."""
     lib = library()
     rng = np.random.default_rng(M + N + K)
@@ -390,6 +390,16 @@ def test_256x128_tiles_rows_sampled(orc, M, N, K, residual):
                              r.data_ptr() if residual else None, N if residual else 0, None, 0))
     sync()
     assert torch.equal(yt, y)  # 32-k stages on the k-strided weight: same products, same summation order
+    # the GELU epilogue (two outputs) on the same tiles
+    y2, g2 = run_fwd(x, w, gelu=True)
+    pre = orc.gemm_fwd(xh[rows], wh)
+    assert rel(host(y2)[rows], pre) < 1e-2
+    assert rel(host(g2)[rows], orc.gelu_fwd(pre)) < 1e-2
+    gt = torch.empty_like(y)
+    check(lib.tgk_gemm_fwd_t(stream(), M, N, K, x.data_ptr(), K, wt.data_ptr(), N, yt.data_ptr(), N, None, 0,
+                             gt.data_ptr(), N))
+    sync()
+    assert torch.equal(yt, y2) and torch.equal(gt, g2)
     # input gradient: dX[M][K] = dY[M][N] W[N][K], tiled over (M, K) and reduced over N
     dy, dyh = to_bf16_device(rng.standard_normal((M, N)))
     w2, w2h = to_bf16_device(rng.standard_normal((N, K)) / np.sqrt(N))
@@ -399,7 +409,15 @@ def test_256x128_tiles_rows_sampled(orc, M, N, K, residual):
     check(lib.tgk_gemm_dgrad_t(stream(), M, N, K, dy.data_ptr(), N, w2t.data_ptr(), N, dxt.data_ptr(), K, None, 0))
     check(lib.tgk_gemm_dgrad(stream(), M, N, K, dy.data_ptr(), N, w2.data_ptr(), K, dx.data_ptr(), K, None, 0))
     sync()
-    assert rel(host(dxt)[rows], orc.gemm_dgrad(dyh[rows], w2h)) < 1e-2
+    want = orc.gemm_dgrad(dyh[rows], w2h)
+    assert rel(host(dxt)[rows], want) < 1e-2
+    assert torch.equal(dxt, dx)
+    # ... and times GELU' of a saved pre-activation
+    u, uh = to_bf16_device(rng.standard_normal((M, K)))
+    check(lib.tgk_gemm_dgrad_t(stream(), M, N, K, dy.data_ptr(), N, w2t.data_ptr(), N, dxt.data_ptr(), K, u.data_ptr(), K))
+    check(lib.tgk_gemm_dgrad(stream(), M, N, K, dy.data_ptr(), N, w2.data_ptr(), K, dx.data_ptr(), K, u.data_ptr(), K))
+    sync()
+    assert rel(host(dxt)[rows], orc.gelu_bwd(uh[rows], want)) < 1e-2
     assert torch.equal(dxt, dx)
 
 

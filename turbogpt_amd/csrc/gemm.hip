@@ -1611,18 +1611,22 @@ void launch_gemm64(hipStream_t stream, Tile tile, const bf16_t *A, int lda, cons
 // The 256-row kernels take products with a plain or residual epilogue whose tiles fill the compute units a whole
 // number of times (or nearly): one block per unit, nothing to cover a tail or a long epilogue (the GELU epilogues
 // stay with gemm64_kernel, where the second block of a unit multiplies meanwhile).
-bool takes_256(int M, int N, int K, int mode, int bn, int k_period) {
-    if (M % 256 || N % bn || K % k_period || (mode != EPI_PLAIN && mode != EPI_RESIDUAL))
+bool takes_256(int M, int N, int K, int bn, int k_period) {
+    if (M % 256 || N % bn || K % k_period)
         return false;
     const int tiles = (M / 256) * (N / bn), units = compute_units();
     const int rounds = (tiles + units - 1) / units;
     return tiles * 10 >= rounds * units * 9; // at least 90 % of the last round filled
 }
 bool takes_256x192(int M, int N, int K, int mode) {
-    return takes_256(M, N, K, mode, 192, 384);
+    return (mode == EPI_PLAIN || mode == EPI_RESIDUAL) && takes_256(M, N, K, 192, 384);
 }
-bool takes_256x128(int M, int N, int K, int mode) { // where the 192-wide tile does not fit
-    return !takes_256x192(M, N, K, mode) && takes_256(M, N, K, mode, 128, 256);
+// Where the 192-wide tile does not fit, with every epilogue: what the 128-wide tile competes with there is two
+// 128 x 128 blocks per unit, and its fewer operand bytes per flop outweigh the uncovered GELU epilogue (measured at
+// d_model 1024: +17 % and +19 % on the two GELU launches; at widths the 192-wide tiles take, gemm64_kernel's 128 x 192
+// blocks keep them)
+bool takes_256x128(int M, int N, int K) {
+    return !takes_256(M, N, K, 192, 384) && takes_256(M, N, K, 128, 256);
 }
 template <int BN = 192, int RA = 3, class Epilogue>
 void launch_gemm256(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
@@ -1654,10 +1658,16 @@ void launch_gemm256_bf16(hipStream_t stream, const bf16_t *A, int lda, const bf1
 // 256 x 128 tiles, A ring of four slots (period of four stages: reduced dimensions that 256 divides)
 void launch_gemm256x128_bf16(hipStream_t stream, const bf16_t *A, int lda, const bf16_t *B, int ldb, int M, int N, int K,
                              const EpilogueBf16 &e) {
-    if (e.mode == EPI_RESIDUAL)
-        launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_RESIDUAL>{e});
-    else
-        launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_PLAIN>{e});
+    switch (e.mode) {
+    case EPI_RESIDUAL:
+        return launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_RESIDUAL>{e});
+    case EPI_GELU:
+        return launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_GELU>{e});
+    case EPI_GELU_BWD:
+        return launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_GELU_BWD>{e});
+    default:
+        return launch_gemm256<128, 4>(stream, A, lda, B, ldb, M, N, K, EpilogueBf16As<EPI_PLAIN>{e});
+    }
 }
 
 // bf16 epilogues of the 64-k kernel: one instantiation per mode
@@ -1715,7 +1725,7 @@ extern "C" int tgk_gemm_fwd(hipStream_t stream, int M, int N, int K, const uint1
         }
         if (takes_256x192(M, N, K, e.mode))
             launch_gemm256_bf16(stream, X, ldx, W, ldw, M, N, K, e);
-        else if (takes_256x128(M, N, K, e.mode))
+        else if (takes_256x128(M, N, K))
             launch_gemm256x128_bf16(stream, X, ldx, W, ldw, M, N, K, e);
         else if (takes_64(tile, K))
             launch_gemm64_bf16<true, true>(stream, tile, X, ldx, W, ldw, M, N, K, e);
@@ -1789,7 +1799,7 @@ extern "C" int tgk_gemm_dgrad_t(hipStream_t stream, int M, int N, int K, const u
         // C[m][i] = sum_o dY[m][o] Wt[i][o]: the forward product with (rows, reduced) = (K, N)
         if (takes_256x192(M, K, N, e.mode))
             launch_gemm256_bf16(stream, dY, lddy, Wt, ldwt, M, K, N, e);
-        else if (takes_256x128(M, K, N, e.mode))
+        else if (takes_256x128(M, K, N))
             launch_gemm256x128_bf16(stream, dY, lddy, Wt, ldwt, M, K, N, e);
         else if (takes_64(tile, N))
             launch_gemm64_bf16<true, true>(stream, tile, dY, lddy, Wt, ldwt, M, K, N, e);
