@@ -226,7 +226,7 @@ def kernel_sweeps(out):
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
         check(lib.tgk_gemm_wgrad_list_prepare(M, len(shapes), ctypes.addressof(jobs), table.data_ptr(), table_bytes))
         ms = timed(lambda: check(lib.tgk_gemm_wgrad_list(stream, M, len(shapes), ctypes.addressof(jobs), table.data_ptr(),
-                                                         0, ws.data_ptr(), need)), iters=5)
+                                                         0, ws.data_ptr(), need, None)), iters=5)
         flop = sum(2.0 * M * n * k for n, k in shapes)
         print(json.dumps({"kernel": "gemm_wgrad_list", "M": M, "jobs": len(shapes), "ms": round(ms, 4),
                           "tflops": round(flop / ms / 1e9, 1),
@@ -250,7 +250,7 @@ def kernel_sweeps(out):
         if table_bytes:
             check(lib.tgk_gemm_wgrad_list_prepare(reduced, 1, ctypes.addressof(one), table.data_ptr(), table_bytes))
             ms = timed(lambda: check(lib.tgk_gemm_wgrad_list(stream, reduced, 1, ctypes.addressof(one), table.data_ptr(), 0,
-                                                             ws.data_ptr(), need)), iters=10)
+                                                             ws.data_ptr(), need, None)), iters=10)
             line["tflops"] = round(flop / ms / 1e9, 1)
         ms = timed(lambda: torch.matmul(a.t(), b), iters=10)
         line["vendor_library_tflops"] = round(flop / ms / 1e9, 1)

@@ -108,7 +108,11 @@ TGK_API size_t tgk_gemm_wgrad_list_table_bytes(int M, int count, const TgkWgradJ
 TGK_API size_t tgk_gemm_wgrad_list_workspace(int M, int count, const TgkWgradJob *jobs);
 TGK_API int tgk_gemm_wgrad_list_prepare(int M, int count, const TgkWgradJob *jobs, void *table, size_t table_bytes);
 TGK_API int tgk_gemm_wgrad_list(hipStream_t stream, int M, int count, const TgkWgradJob *jobs, const void *table,
-                                int accumulate, void *workspace, size_t workspace_bytes);
+                                int accumulate, void *workspace, size_t workspace_bytes, float *sumsq);
+/* `sumsq` (may be NULL) receives tgk_gemm_wgrad_list_sumsq_count floats whose sum is the sum of squares of every
+ * gradient element the call writes: the kernels that write a gradient square it on the way, in a fixed order, so that
+ * the clip norm (cuda/trainer.cuh:35-46, cuda/optim.cuh:67-80) needs no second pass over these matrices. */
+TGK_API int tgk_gemm_wgrad_list_sumsq_count(int M, int count, const TgkWgradJob *jobs);
 
 
 /* ---- Causal softmax attention, head_dim 64.  Takes the slot of attention_forward /
@@ -207,6 +211,10 @@ TGK_API int tgk_transpose_batch(hipStream_t stream, const uint16_t *in, uint16_t
 
 /* partials[i] = sum of squares of block i's share of g (cuda/trainer.cuh:35-46); count <= 4096. */
 TGK_API int tgk_sumsq_partials(hipStream_t stream, const float *g, size_t n, float *partials, int count);
+/* partials[i] = sum of squares of g[start_i .. start_i + length_i): the same for a list of ranges, one block each
+ * (the tensors whose gradients tgk_gemm_wgrad_list does not write, cut into ranges of a few thousand elements).
+ * segments: device array of {int64 start, length}, both multiples of 4; count <= 4096. */
+TGK_API int tgk_sumsq_segments(hipStream_t stream, const float *g, const void *segments, int count, float *partials);
 /* AdamW on the hi/lo weight halves (cuda/optim.cuh:67-106): clip scale min(1, clip/(||g||+1e-6))
  * from the folded partials when clip > 0, m += (1-b1)(g-m), v = b2 v + (1-b2) g^2,
  * w = w (1 - lr*wd) - (lr/bc1) m / (sqrt(v)/sqrt(bc2) + eps), bias corrections from `step`

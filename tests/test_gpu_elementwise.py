@@ -176,6 +176,27 @@ def run_adamw(orc, w, m, v, g, bounds, flags, steps, clip, lr=6e-4, wd=0.1):
     return out, md.cpu().numpy(), vd.cpu().numpy()
 
 
+def test_sums_of_squares_over_a_list_of_ranges():
+    """tgk_sumsq_segments: one partial per range, equal to numpy's sum over that range; ranges of every length class
+    (shorter than a block's stride, not a multiple of it, many strides long), NaN outside the ranges."""
+    lib = library()
+    rng = np.random.default_rng(11)
+    g = rng.standard_normal(200_000).astype(np.float32)
+    ranges = [(0, 4), (8, 1536), (4096, 8192), (20_000, 8188), (100_000, 65_536)]
+    masked = np.full_like(g, np.nan)
+    for start, length in ranges:
+        masked[start:start + length] = g[start:start + length]
+    gd = dev(masked)
+    rd = dev(np.asarray(ranges, np.int64))
+    parts = torch.full((len(ranges),), float("nan"), dtype=torch.float32, device="cuda")
+    check(lib.tgk_sumsq_segments(stream(), gd.data_ptr(), rd.data_ptr(), len(ranges), parts.data_ptr()))
+    sync()
+    want = [float((g[a:a + n].astype(np.float64) ** 2).sum()) for a, n in ranges]
+    np.testing.assert_allclose(parts.cpu().numpy(), want, rtol=2e-6)
+    assert lib.tgk_sumsq_segments(stream(), gd.data_ptr(), None, 1, parts.data_ptr()) == -1
+    assert lib.tgk_sumsq_segments(stream(), gd.data_ptr(), rd.data_ptr(), 0, parts.data_ptr()) == -1
+
+
 @pytest.mark.parametrize("clip", [0.0, 1.0])
 def test_adamw_matches_the_checker_over_20_steps(orc, clip):
     # tests/verify.py:64-105 (AdamW part): N(0, 0.01) gradients from default_rng(192)

@@ -250,10 +250,20 @@ def run_wgrad_list(M, shapes, rng, strides=None):
     need = lib.tgk_gemm_wgrad_list_workspace(M, len(shapes), C.addressof(jobs))
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
     check(lib.tgk_gemm_wgrad_list_prepare(M, len(shapes), C.addressof(jobs), table.data_ptr(), table_bytes))
+    # the sums of squares of what the call writes come with it: their total is ||dW||^2 over all jobs
+    count = lib.tgk_gemm_wgrad_list_sumsq_count(M, len(shapes), C.addressof(jobs))
+    assert 0 < count <= 4096
+    squares = torch.full((count,), float("nan"), dtype=torch.float32, device="cuda")
     call = lambda: check(lib.tgk_gemm_wgrad_list(stream(), M, len(shapes), C.addressof(jobs), table.data_ptr(), 0,
-                                                 ws.data_ptr(), need))
+                                                 ws.data_ptr(), need, squares.data_ptr()))
     call()
     sync()
+    written = sum(float((dw.double()[:, :K] ** 2).sum()) for (dy, x, dw), (N, K) in zip(keep, shapes))
+    assert abs(float(squares.double().sum()) - written) <= 1e-5 * written
+    first = squares.clone()
+    call()
+    sync()
+    assert torch.equal(first, squares)  # fixed order: bit-reproducible
     return keep, inputs, (jobs, table, ws, call)
 
 
@@ -331,10 +341,10 @@ def test_wgrad_list_rejects_bad_jobs():
     assert b"table too small" in lib.tgk_error()
     check(lib.tgk_gemm_wgrad_list_prepare(128, 1, C.addressof(jobs), f.data_ptr(), 1 << 16))
     ws = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
-    assert lib.tgk_gemm_wgrad_list(stream(), 128, 1, C.addressof(jobs), f.data_ptr(), 1, ws.data_ptr(), 1 << 20) == -1
+    assert lib.tgk_gemm_wgrad_list(stream(), 128, 1, C.addressof(jobs), f.data_ptr(), 1, ws.data_ptr(), 1 << 20, None) == -1
     assert b"accumulate" in lib.tgk_error()
-    assert lib.tgk_gemm_wgrad_list(stream(), 128, 1, C.addressof(jobs), None, 0, ws.data_ptr(), 1 << 20) == -1
-    assert lib.tgk_gemm_wgrad_list(stream(), 128, 0, C.addressof(jobs), f.data_ptr(), 0, ws.data_ptr(), 1 << 20) == -1
+    assert lib.tgk_gemm_wgrad_list(stream(), 128, 1, C.addressof(jobs), None, 0, ws.data_ptr(), 1 << 20, None) == -1
+    assert lib.tgk_gemm_wgrad_list(stream(), 128, 0, C.addressof(jobs), f.data_ptr(), 0, ws.data_ptr(), 1 << 20, None) == -1
     sync()
 
 

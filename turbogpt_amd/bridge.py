@@ -28,7 +28,8 @@ KERNEL_ABI = {
     "tgk_gemm_wgrad_list_table_bytes": (sz, [i32, i32, vp]),
     "tgk_gemm_wgrad_list_workspace": (sz, [i32, i32, vp]),
     "tgk_gemm_wgrad_list_prepare": (i32, [i32, i32, vp, vp, sz]),
-    "tgk_gemm_wgrad_list": (i32, [vp, i32, i32, vp, vp, i32, vp, sz]),
+    "tgk_gemm_wgrad_list": (i32, [vp, i32, i32, vp, vp, i32, vp, sz, vp]),
+    "tgk_gemm_wgrad_list_sumsq_count": (i32, [i32, i32, vp]),
     "tgk_attn_fwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, f32]),
     "tgk_attn_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, i32, vp, i32, vp, vp, i32, vp, vp, vp, i32,
                            f32, vp, sz]),
@@ -47,6 +48,7 @@ KERNEL_ABI = {
     "tgk_layernorm_bwd_fold": (i32, [vp, i32, i32, i32, vp, sz, vp, i32]),
     "tgk_cross_entropy": (i32, [vp, i32, i32, vp, vp, vp, vp, f32, i32]),
     "tgk_sumsq_partials": (i32, [vp, vp, sz, vp, i32]),
+    "tgk_sumsq_segments": (i32, [vp, vp, vp, i32, vp]),
     "tgk_adamw": (i32, [vp, sz, vp, vp, vp, vp, vp, vp, i32, vp, vp, i32, f32, f32, f32, f32, f32, f32,
                         C.c_uint64]),
     "tgk_sample_batch": (i32, [vp, vp, i64, C.c_uint64, C.c_uint64, i32, i32, vp, vp]),

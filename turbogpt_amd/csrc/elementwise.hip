@@ -490,6 +490,32 @@ __global__ __launch_bounds__(256) void sumsq_kernel(const float *__restrict__ g,
         partial[blockIdx.x] = (waves[0] + waves[1]) + (waves[2] + waves[3]);
 }
 
+// The same for a list of ranges of g, one block per range (the parameter tensors whose gradients no matrix kernel
+// writes: the caller cuts long tensors into ranges of a few thousand elements).  Starts and lengths multiples of 4.
+struct SumsqSegment {
+    int64_t start, length;
+};
+__global__ __launch_bounds__(256) void sumsq_segments_kernel(const float *__restrict__ g,
+                                                             const SumsqSegment *__restrict__ segments,
+                                                             float *__restrict__ partial) {
+    __shared__ float waves[4];
+    const SumsqSegment segment = segments[blockIdx.x];
+    const f32x4 *p = reinterpret_cast<const f32x4 *>(g + segment.start);
+    const int quads = int(segment.length >> 2);
+    float sum = 0.f;
+#pragma unroll 8
+    for (int i = threadIdx.x; i < quads; i += 256) {
+        const f32x4 v = p[i];
+        sum += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+    sum = wave_sum(sum);
+    if ((threadIdx.x & 63) == 0)
+        waves[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0)
+        partial[blockIdx.x] = (waves[0] + waves[1]) + (waves[2] + waves[3]);
+}
+
 struct AdamArgs {
     float lr, beta1, beta2, eps, weight_decay, bc1, sqrt_bc2, clip;
 };
@@ -868,6 +894,16 @@ extern "C" int tgk_sumsq_partials(hipStream_t stream, const float *g, size_t n, 
     });
 }
 
+extern "C" int tgk_sumsq_segments(hipStream_t stream, const float *g, const void *segments, int count, float *partials) {
+    return guarded([&] {
+        aligned(g, "sumsq_segments: g");
+        require(segments && !(reinterpret_cast<uintptr_t>(segments) & 7) && partials && count > 0 && count <= 4096,
+                "sumsq_segments: 1..4096 ranges in a device array, and their partials");
+        hipLaunchKernelGGL(sumsq_segments_kernel, dim3(count), dim3(256), 0, stream, g,
+                           static_cast<const SumsqSegment *>(segments), partials);
+        check_hip(hipGetLastError(), "sumsq_segments launch: ");
+    });
+}
 extern "C" int tgk_adamw(hipStream_t stream, size_t n, uint16_t *weight_hi, uint16_t *weight_lo, float *m,
                          float *v, const float *g, const float *norm_partials, int norm_count,
                          const int64_t *segment_starts, const uint8_t *segment_flags, int segments,

@@ -76,6 +76,11 @@ struct Slot {
     std::vector<bf16_t *> g_x, g_mid, g_u, g_qkv;
     std::vector<TgkWgradJob> wgrad_jobs;
     void *wgrad_table = nullptr;
+    // ... and the kernels that write the gradient leave the sums of its squares here (cuda/trainer.cuh:35-46): the
+    // launch above for the matrices, one more small launch for the ranges in `norm_ranges` (every other tensor)
+    float *norms = nullptr;
+    int list_norms = 0, range_norms = 0;
+    void *norm_ranges = nullptr;
     void *workspace = nullptr;
     // LayerNorm parameter gradients: every LayerNorm backward of a step leaves its per-block partial sums in a
     // block of its own here and one launch at the end of the backward pass folds all 2 * depth + 1 of them
@@ -311,8 +316,11 @@ struct Engine {
             OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_fold(stream, M, d, 2 * c.depth + 1, s.ln_partials, ln_stride, s.ln_targets, 0));
             OP(TG_CLASS_OTHER, tgk_embed_bwd(stream, c.batch, T, d, V, tokens_in, s.g_x[0], g + layout.embedding,
                                              g + layout.positions, 0, workspace, workspace_bytes));
+            const bool norms = c.clip > 0;
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad_list(stream, M, int(s.wgrad_jobs.size()), s.wgrad_jobs.data(), s.wgrad_table, 0,
-                                                        workspace, workspace_bytes));
+                                                        workspace, workspace_bytes, norms ? s.norms : nullptr));
+            if (norms)
+                OP(TG_CLASS_OPTIMIZER, tgk_sumsq_segments(stream, g, s.norm_ranges, s.range_norms, s.norms + s.list_norms));
             return;
         }
         OP(TG_CLASS_HEAD, tgk_gemm_wgrad(stream, M, V, d, logits, V, nf, d, g + layout.head, d, 0, workspace, workspace_bytes));
@@ -364,7 +372,8 @@ struct Engine {
 
     // cuda/optim.cuh:66-106 for optimizer step `at` (0-based), on the engine's stream: gradient -> the weights of
     // version `to` (which already hold the previous version's values)
-    void optimize(uint64_t at, const float *gradient, Version &to) {
+    // `from`: the slot whose backward pass has just written `gradient`, when it left the sums of squares with it
+    void optimize(uint64_t at, const float *gradient, Version &to, const Slot *from = nullptr) {
         const Config &c = config.base;
         uint16_t *weight_hi = to.hi, *weight_lo = to.lo, *weight_t = to.t;
         float lr = c.learning_rate, beta1 = c.beta1, muon_lr = c.muon_lr, muon_momentum = c.momentum;
@@ -373,11 +382,12 @@ struct Engine {
             muon_lr *= schedule[at].multiplier;
             beta1 = muon_momentum = schedule[at].momentum;
         }
-        if (c.clip > 0)
+        const bool fused = from && from->norms && list_wgrad;
+        if (c.clip > 0 && !fused)
             OP(TG_CLASS_OPTIMIZER, tgk_sumsq_partials(stream, gradient, size_t(layout.count), norm_partials, NormPartials));
         OP(TG_CLASS_OPTIMIZER, tgk_adamw(stream, size_t(layout.count), weight_hi, weight_lo, momentum, variance, gradient,
-                     norm_partials, NormPartials, segment_starts, segment_flags, segments, lr, beta1, c.beta2,
-                     c.epsilon, c.weight_decay, c.clip, at));
+                     fused ? from->norms : norm_partials, fused ? from->list_norms + from->range_norms : NormPartials,
+                     segment_starts, segment_flags, segments, lr, beta1, c.beta2, c.epsilon, c.weight_decay, c.clip, at));
         if (width16) { // the hidden matrices, which the AdamW segments skip (cuda/optim.cuh:107-118)
             OP(TG_CLASS_OPTIMIZER, tgk_w16_muon(stream, c.depth, weight_hi, weight_lo, momentum, gradient, norm_partials,
                                                 NormPartials, c.clip, muon_lr, muon_momentum, c.weight_decay, c.ns_steps));
@@ -405,7 +415,7 @@ struct Engine {
         const uint64_t K = slots.size(), ring = versions.size();
         if (K == 1) {
             batch_gradient(slots[0], versions[0], at, history_row);
-            optimize(at, slots[0].gradient, versions[0]);
+            optimize(at, slots[0].gradient, versions[0], &slots[0]);
             *trace = int(at);
             return;
         }
@@ -419,7 +429,7 @@ struct Engine {
         const size_t bytes = size_t(layout.count) * 2;
         check_hip(hipMemcpyAsync(to.hi, from.hi, bytes, hipMemcpyDeviceToDevice, stream));
         check_hip(hipMemcpyAsync(to.lo, from.lo, bytes, hipMemcpyDeviceToDevice, stream));
-        optimize(at, s.gradient, to);
+        optimize(at, s.gradient, to, &s);
         check_hip(hipEventRecord(to.done, stream));
         *trace = int(read);
         total_staleness += at - read;
@@ -734,6 +744,38 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
                 e->allocate(table, table_bytes, false);
                 slot.wgrad_table = table;
                 ok(tgk_gemm_wgrad_list_prepare(int(M), int(slot.wgrad_jobs.size()), slot.wgrad_jobs.data(), table, table_bytes));
+                // the tensors no matrix product writes, in ranges of at most 8192 elements; with the matrices they
+                // must cover the flat gradient exactly
+                struct Range {
+                    int64_t start, length;
+                };
+                std::vector<Range> ranges;
+                int64_t covered = int64_t(V) * d; // the head
+                const auto cover = [&](int64_t start, int64_t length) {
+                    covered += length;
+                    for (int64_t at = 0; at < length; at += 8192)
+                        ranges.push_back({start + at, std::min<int64_t>(8192, length - at)});
+                };
+                cover(e->layout.embedding, int64_t(V) * d);
+                cover(e->layout.positions, int64_t(c.context) * d);
+                for (int l = 0; l < c.depth; ++l) {
+                    const TgLayerParameters &p = e->layout.layers[l];
+                    cover(p.ln1_g, d), cover(p.ln1_b, d), cover(p.ln2_g, d), cover(p.ln2_b, d);
+                    covered += 4 * int64_t(d) * d + 2 * int64_t(F) * d;
+                }
+                cover(e->layout.lnf_g, d), cover(e->layout.lnf_b, d);
+                if (covered != e->layout.count)
+                    throw std::runtime_error("engine: gradient norm ranges do not cover the parameters");
+                slot.list_norms = tgk_gemm_wgrad_list_sumsq_count(int(M), int(slot.wgrad_jobs.size()), slot.wgrad_jobs.data());
+                slot.range_norms = int(ranges.size());
+                if (slot.list_norms <= 0 || slot.list_norms + slot.range_norms > 4096)
+                    throw std::runtime_error("engine: too many gradient norm partials");
+                e->allocate(slot.norms, size_t(slot.list_norms + slot.range_norms), false);
+                uint8_t *device_ranges = nullptr;
+                e->allocate(device_ranges, ranges.size() * sizeof(Range), false);
+                check_hip(hipMemcpy(device_ranges, ranges.data(), ranges.size() * sizeof(Range), hipMemcpyHostToDevice),
+                          "norm ranges: ");
+                slot.norm_ranges = device_ranges;
                 batch_need = std::max(batch_need, tgk_gemm_wgrad_list_workspace(int(M), int(slot.wgrad_jobs.size()), slot.wgrad_jobs.data()));
             }
         }

@@ -1222,6 +1222,8 @@ struct WgradList {
     int k_quads;              // tokens / 128
     int accumulate;
     float *pieces; // rem_tiles * rem_splits partial tiles of 256 * BN floats, row major
+    float *sumsq;  // optional: sums of squares of the gradients written, four per block of the product launch (one per
+                   // wave) followed by one per block of the fold launch
 };
 struct WgradListItem {
     int tile, q0, nq, piece; // piece < 0: the block reduces over all tokens and writes the gradient itself
@@ -1401,6 +1403,7 @@ __global__ __launch_bounds__(256, 1) void wgrad_list_kernel(const WgradList w) {
     int index = 0;
     wgrad_list_item(w, 0, item);
     int quads_left = item.nq;
+    float squares = 0.f; // of the gradient elements this lane has written (not of pieces: the fold squares their sums)
     clear();
     for (;;) {
         step(std::integral_constant<int, 0>{}, fa0, fb0, fa1, fb1);
@@ -1426,6 +1429,23 @@ __global__ __launch_bounds__(256, 1) void wgrad_list_kernel(const WgradList w) {
             out += size_t(16) * ld;
             asm volatile("" : "+v"(out));
         }
+        // the squares of what went out, one 16 x 16 tile at a time (fenced: all 256 accumulators read at once do not
+        // fit beside the fragments)
+        if (w.sumsq && item.piece < 0) {
+#pragma unroll
+            for (int i = 0; i < AF; ++i)
+#pragma unroll
+                for (int j = 0; j < BF; ++j) {
+                    // read through assembly: an accumulator that plain code reads stops being pinned to the
+                    // accumulation registers, and the allocation of the whole kernel falls apart (103 spills)
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[e]) : "a"(acc[i >> 1][j >> 1][i & 1][j & 1][e]));
+                    squares += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        }
         // the copy counter must hold nothing but the three stages the steps assume: let the stores drain
         wait_vmcnt<0>();
         if (!wgrad_list_item(w, ++index, item))
@@ -1434,10 +1454,18 @@ __global__ __launch_bounds__(256, 1) void wgrad_list_kernel(const WgradList w) {
         clear();
     }
     wait_vmcnt<0>();
+    if (w.sumsq) { // fixed tiles per block, fixed order inside a lane and inside a wave: bit-reproducible
+        squares = wave_sum(squares);
+        if (lane == 0)
+            w.sumsq[blockIdx.x * 4 + wave] = squares;
+    }
 }
 // Sums the pieces of the split tiles, in token order, into the gradient.  Eight blocks per tile.
-template <int BN> __global__ __launch_bounds__(256) void wgrad_list_fold_kernel(const WgradList w, int first_tile) {
+template <int BN>
+__global__ __launch_bounds__(256) void wgrad_list_fold_kernel(const WgradList w, int first_tile, int first_sumsq) {
     constexpr int BM = 256, QUADS = BM * BN / 4 / 8 / 256; // float4 per thread
+    __shared__ float waves[4];
+    float squares = 0.f;
     const int r = blockIdx.x >> 3, part = blockIdx.x & 7;
     const int4 t = w.tiles[first_tile + r];
     const WgradListJob job = w.jobs[t.x];
@@ -1453,6 +1481,15 @@ template <int BN> __global__ __launch_bounds__(256) void wgrad_list_fold_kernel(
         if (w.accumulate)
             sum += *p;
         __builtin_nontemporal_store(sum, p);
+        squares += (sum[0] * sum[0] + sum[1] * sum[1]) + (sum[2] * sum[2] + sum[3] * sum[3]);
+    }
+    if (w.sumsq) {
+        squares = wave_sum(squares);
+        if ((threadIdx.x & 63) == 0)
+            waves[threadIdx.x >> 6] = squares;
+        __syncthreads();
+        if (threadIdx.x == 0)
+            w.sumsq[first_sumsq + blockIdx.x] = (waves[0] + waves[1]) + (waves[2] + waves[3]);
     }
 }
 
@@ -1959,7 +1996,7 @@ extern "C" int tgk_gemm_wgrad_batch(hipStream_t stream, int M, int count, const 
 namespace {
 // Tables and split of a whole-step weight-gradient launch.
 struct WgradListPlan {
-    int tiles, blocks, rounds, rem_tiles, rem_splits;
+    int tiles, blocks, rounds, rem_tiles, rem_splits, launch_blocks, fold_blocks;
     size_t jobs_bytes, table_bytes, pieces_bytes;
 };
 bool plan_wgrad_list(int M, int count, const TgkWgradJob *jobs, WgradListPlan &plan, std::string &why) {
@@ -1988,6 +2025,8 @@ bool plan_wgrad_list(int M, int count, const TgkWgradJob *jobs, WgradListPlan &p
     plan.jobs_bytes = (size_t(count) * sizeof(WgradListJob) + 15) / 16 * 16;
     plan.table_bytes = plan.jobs_bytes + size_t(tiles) * sizeof(int4);
     plan.pieces_bytes = plan.rem_splits > 1 ? size_t(plan.rem_tiles) * plan.rem_splits * 256 * 256 * sizeof(float) : 0;
+    plan.launch_blocks = plan.rounds ? plan.blocks : plan.rem_tiles * plan.rem_splits;
+    plan.fold_blocks = plan.rem_splits > 1 ? plan.rem_tiles * 8 : 0;
     return true;
 }
 } // namespace
@@ -2006,6 +2045,15 @@ extern "C" size_t tgk_gemm_wgrad_list_workspace(int M, int count, const TgkWgrad
         WgradListPlan plan;
         std::string why;
         return plan_wgrad_list(M, count, jobs, plan, why) ? plan.pieces_bytes : 0;
+    } catch (...) {
+        return 0;
+    }
+}
+extern "C" int tgk_gemm_wgrad_list_sumsq_count(int M, int count, const TgkWgradJob *jobs) {
+    try {
+        WgradListPlan plan;
+        std::string why;
+        return plan_wgrad_list(M, count, jobs, plan, why) ? 4 * plan.launch_blocks + plan.fold_blocks : 0;
     } catch (...) {
         return 0;
     }
@@ -2038,7 +2086,7 @@ extern "C" int tgk_gemm_wgrad_list_prepare(int M, int count, const TgkWgradJob *
     });
 }
 extern "C" int tgk_gemm_wgrad_list(hipStream_t stream, int M, int count, const TgkWgradJob *jobs, const void *table,
-                                   int accumulate, void *workspace, size_t workspace_bytes) {
+                                   int accumulate, void *workspace, size_t workspace_bytes, float *sumsq) {
     return guarded([&] {
         WgradListPlan plan;
         std::string why;
@@ -2056,6 +2104,8 @@ extern "C" int tgk_gemm_wgrad_list(hipStream_t stream, int M, int count, const T
         w.k_quads = M / 128;
         w.accumulate = accumulate;
         w.pieces = static_cast<float *>(workspace);
+        require(!(reinterpret_cast<uintptr_t>(sumsq) & 3), "gemm_wgrad_list: sumsq must be 4-byte aligned");
+        w.sumsq = sumsq;
         auto kernel = wgrad_list_kernel<256>;
         constexpr size_t lds = 4 * (256 + 256) * 64;
         static std::atomic<bool> configured[MAX_DEVICES];
@@ -2066,12 +2116,11 @@ extern "C" int tgk_gemm_wgrad_list(hipStream_t stream, int M, int count, const T
                       "gemm LDS size: ");
             configured[device].store(true, std::memory_order_release);
         }
-        const int blocks = plan.rounds ? plan.blocks : plan.rem_tiles * plan.rem_splits;
-        hipLaunchKernelGGL(kernel, dim3(blocks), dim3(256), lds, stream, w);
+        hipLaunchKernelGGL(kernel, dim3(plan.launch_blocks), dim3(256), lds, stream, w);
         check_hip(hipGetLastError(), "wgrad list launch: ");
-        if (plan.rem_splits > 1) {
-            hipLaunchKernelGGL((wgrad_list_fold_kernel<256>), dim3(plan.rem_tiles * 8), dim3(256), 0, stream, w,
-                               plan.rounds * plan.blocks);
+        if (plan.fold_blocks) {
+            hipLaunchKernelGGL((wgrad_list_fold_kernel<256>), dim3(plan.fold_blocks), dim3(256), 0, stream, w,
+                               plan.rounds * plan.blocks, 4 * plan.launch_blocks);
             check_hip(hipGetLastError(), "wgrad list fold launch: ");
         }
     });
