@@ -163,6 +163,11 @@ TGK_API int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab, co
                           const uint16_t *dh, float *dtable, float *dpositions, int accumulate,
                           void *workspace, size_t workspace_bytes);
 TGK_API size_t tgk_embed_bwd_workspace(int rows, int D);
+/* The same in two parts, for a caller that multiplies weight gradients as one list (tgk_gemm_wgrad_list): writes the
+ * exact one-hot matrix of the tokens, onehot[B*T][256] (bf16, 16-byte aligned), whose product onehot^T . dh IS dtable -
+ * one more job {N = 256, K = D, dY = onehot, X = dh} of that list - and computes dpositions as above. */
+TGK_API int tgk_embed_bwd_onehot(hipStream_t stream, int B, int T, int D, const uint8_t *x, const uint16_t *dh,
+                                 uint16_t *onehot, float *dpositions, int accumulate);
 
 /* y = RN_bf16((x - mean) * rsqrt(var + eps) * gamma + beta) per row; takes the slot of normalize
  * (cuda/ops.cuh:57-66; RMSNorm there, LayerNorm in the target model). D multiple of 8, <= 2048. */

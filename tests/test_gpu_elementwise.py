@@ -51,6 +51,18 @@ def test_embedding_forward_and_backward(orc, B, T, D):
                             ws.data_ptr(), need))
     sync()
     assert rel(host(dt), 2 * want_t) < 1e-6
+    # the two-part form: the exact one-hot matrix (its product with dh is the table gradient) and the same positions
+    onehot = torch.full((B * T, 256), 7.0, dtype=torch.bfloat16, device="cuda")
+    dp2 = torch.full((T, D), 1.0, dtype=torch.float32, device="cuda")
+    check(lib.tgk_embed_bwd_onehot(stream(), B, T, D, xd.data_ptr(), dh.data_ptr(), onehot.data_ptr(), dp2.data_ptr(), 0))
+    sync()
+    want_hot = np.zeros((B * T, 256), np.float32)
+    want_hot[np.arange(B * T), x] = 1.0
+    np.testing.assert_array_equal(onehot.float().cpu().numpy(), want_hot)
+    check(lib.tgk_embed_bwd(stream(), B, T, D, 256, xd.data_ptr(), dh.data_ptr(), dt.data_ptr(), dp.data_ptr(), 0,
+                            ws.data_ptr(), need))
+    sync()
+    assert torch.equal(dp2, dp)
 
 
 @pytest.mark.parametrize("M,D", [(64, 256), (333, 768), (128, 1024), (16, 2048)])

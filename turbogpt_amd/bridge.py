@@ -40,6 +40,7 @@ KERNEL_ABI = {
     "tgk_embed_fwd": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
     "tgk_embed_bwd": (i32, [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32, vp, sz]),
     "tgk_embed_bwd_workspace": (sz, [i32, i32]),
+    "tgk_embed_bwd_onehot": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, i32]),
     "tgk_layernorm_fwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, f32]),
     "tgk_layernorm_bwd": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, f32, i32, i32, vp, sz]),
     "tgk_layernorm_bwd_add": (i32, [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, f32, i32, vp, sz]),

@@ -704,6 +704,19 @@ extern "C" size_t tgk_embed_bwd_workspace(int rows, int D) {
         return onehot_bytes(rows) + tgk_gemm_wgrad_workspace(rows, 256, D);
     return size_t((rows + EMBED_SEGMENT - 1) / EMBED_SEGMENT) * 256 * D * sizeof(float);
 }
+extern "C" int tgk_embed_bwd_onehot(hipStream_t stream, int B, int T, int D, const uint8_t *x, const uint16_t *dh,
+                                    uint16_t *onehot, float *dpositions, int accumulate) {
+    return guarded([&] {
+        require(B > 0 && T > 0 && D > 0 && D % 64 == 0, "embed_bwd_onehot: D must be a positive multiple of 64");
+        require(x && dh && dpositions, "embed_bwd_onehot: missing operand");
+        aligned(onehot, "embed_bwd_onehot: onehot");
+        const int rows = B * T;
+        hipLaunchKernelGGL(onehot_kernel, dim3(grid_for(size_t(rows) * 32, 256)), dim3(256), 0, stream, x, onehot, rows);
+        hipLaunchKernelGGL(embed_bwd_positions_kernel, dim3(grid_for(size_t(T) * D, 256)), dim3(256), 0, stream,
+                           dh, dpositions, B, T, D, accumulate);
+        check_hip(hipGetLastError(), "embed_bwd_onehot launch: ");
+    });
+}
 extern "C" int tgk_embed_bwd(hipStream_t stream, int B, int T, int D, int vocab, const uint8_t *x,
                              const uint16_t *dh, float *dtable, float *dpositions, int accumulate,
                              void *workspace, size_t workspace_bytes) {

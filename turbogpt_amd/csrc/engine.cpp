@@ -76,6 +76,7 @@ struct Slot {
     std::vector<bf16_t *> g_x, g_mid, g_u, g_qkv;
     std::vector<TgkWgradJob> wgrad_jobs;
     void *wgrad_table = nullptr;
+    bf16_t *onehot = nullptr; // [tokens][256]: the token table's gradient is one more product of that launch
     // ... and the kernels that write the gradient leave the sums of its squares here (cuda/trainer.cuh:35-46): the
     // launch above for the matrices, one more small launch for the ranges in `norm_ranges` (every other tensor)
     float *norms = nullptr;
@@ -295,8 +296,8 @@ struct Engine {
         };
         if (list_wgrad) {
             // No weight gradient in the loop: every block leaves its output gradients in buffers of its own and one
-            // launch at the end computes all 4 * depth + 1 products (the head's included; its operands are dlogits,
-            // still in `logits`, and nf).
+            // launch at the end computes all 4 * depth + 2 products (the head's included - its operands are dlogits,
+            // still in `logits`, and nf - and the token table's, one-hot^T times the gradient entering the first block).
             OP(TG_CLASS_HEAD, tgk_gemm_dgrad_t(stream, M, V, d, logits, V, wt(layout.head), V, t1, d, nullptr, 0));
             OP(TG_CLASS_LAYERNORM_BWD, ln_rows(0, x[c.depth], t1, layout.lnf_g, nullptr, s.g_x[c.depth]));
             for (int l = c.depth - 1; l >= 0; --l) {
@@ -314,8 +315,7 @@ struct Engine {
                 OP(TG_CLASS_LAYERNORM_BWD, ln_rows(2 + 2 * l, x[l], t1, p.ln1_g, mid, s.g_x[l]));
             }
             OP(TG_CLASS_LAYERNORM_BWD, tgk_layernorm_bwd_fold(stream, M, d, 2 * c.depth + 1, s.ln_partials, ln_stride, s.ln_targets, 0));
-            OP(TG_CLASS_OTHER, tgk_embed_bwd(stream, c.batch, T, d, V, tokens_in, s.g_x[0], g + layout.embedding,
-                                             g + layout.positions, 0, workspace, workspace_bytes));
+            OP(TG_CLASS_OTHER, tgk_embed_bwd_onehot(stream, c.batch, T, d, tokens_in, s.g_x[0], s.onehot, g + layout.positions, 0));
             const bool norms = c.clip > 0;
             OP(TG_CLASS_GEMM_WGRAD, tgk_gemm_wgrad_list(stream, M, int(s.wgrad_jobs.size()), s.wgrad_jobs.data(), s.wgrad_table, 0,
                                                         workspace, workspace_bytes, norms ? s.norms : nullptr));
@@ -715,7 +715,8 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
             for (int l = 0; l < c.depth; ++l)
                 for (int j = 0; j < 4; ++j)
                     jobs.push_back(block_jobs[j]);
-            jobs.push_back({int(V), int(d), nullptr, int(V), nullptr, int(d), nullptr, int(d)});
+            jobs.push_back({int(V), int(d), nullptr, int(V), nullptr, int(d), nullptr, int(d)}); // the head
+            jobs.push_back({int(V), int(d), nullptr, int(V), nullptr, int(d), nullptr, int(d)}); // the token table
             table_bytes = tgk_gemm_wgrad_list_table_bytes(int(M), int(jobs.size()), jobs.data());
         }
         e->list_wgrad = table_bytes > 0;
@@ -738,8 +739,10 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
                     jobs[2].dY = slot.g_mid[l], jobs[2].X = b.o, jobs[2].dW = g + p.attn_out;
                     jobs[3].dY = slot.g_qkv[l], jobs[3].X = b.n1, jobs[3].dW = g + p.qkv;
                 }
-                TgkWgradJob &head = slot.wgrad_jobs.back();
+                TgkWgradJob &head = slot.wgrad_jobs[4 * c.depth], &table_job = slot.wgrad_jobs[4 * c.depth + 1];
                 head.dY = slot.logits, head.X = slot.nf, head.dW = slot.gradient + e->layout.head;
+                e->allocate(slot.onehot, M * V, false);
+                table_job.dY = slot.onehot, table_job.X = slot.g_x[0], table_job.dW = slot.gradient + e->layout.embedding;
                 uint8_t *table = nullptr;
                 e->allocate(table, table_bytes, false);
                 slot.wgrad_table = table;
@@ -750,13 +753,12 @@ TG_API Engine *tg_create_ex(const TgModelConfig *model) {
                     int64_t start, length;
                 };
                 std::vector<Range> ranges;
-                int64_t covered = int64_t(V) * d; // the head
+                int64_t covered = 2 * int64_t(V) * d; // the head and the token table
                 const auto cover = [&](int64_t start, int64_t length) {
                     covered += length;
                     for (int64_t at = 0; at < length; at += 8192)
                         ranges.push_back({start + at, std::min<int64_t>(8192, length - at)});
                 };
-                cover(e->layout.embedding, int64_t(V) * d);
                 cover(e->layout.positions, int64_t(c.context) * d);
                 for (int l = 0; l < c.depth; ++l) {
                     const TgLayerParameters &p = e->layout.layers[l];
