@@ -72,15 +72,17 @@ def class_work():
     act, wide = M * D * 2, M * F * 2
     params = V * D * 2 + T * D + L * (4 * D + 4 * D * D + 2 * F * D) + 2 * D
     qkv, out, up, down = gemm_flops()
+    # widths that 256 divides: one launch computes every weight gradient, the head's and the token table's included
+    listed = 2 if D % 256 == 0 else 0
     return {
         "gemm_fwd": ("flop", L * (qkv + out + down)),     # plain / residual epilogues
         "gemm_fwd_gelu": ("flop", L * up),                # MLP-up: pre-activation and GELU written
         "gemm_dgrad": ("flop", L * (qkv + out + up)),     # plain epilogue
         "gemm_dgrad_gelu": ("flop", L * down),            # MLP-down dgrad times GELU'
-        "gemm_wgrad": ("flop", L * per_layer),
+        "gemm_wgrad": ("flop", L * per_layer + listed * 2.0 * M * V * D),
         "attn_fwd": ("flop", L * attn_fwd),
         "attn_bwd": ("flop", L * attn_fwd * 2.5),
-        "head": ("flop", 3 * 2.0 * M * V * D),
+        "head": ("flop", (3 - listed // 2) * 2.0 * M * V * D),
         "layernorm_fwd": ("byte", (2 * L + 1) * 2 * act),
         "layernorm_bwd": ("byte", (2 * L + 1) * 3 * act + 2 * L * act),  # x, dy, dx (+ residual read)
         "optimizer": ("byte", params * 28.0 + params * 4.0),            # AdamW 28 B/param + norm pass
